@@ -1,0 +1,54 @@
+// Shared helpers of the gfx950 kernels behind include/dmoe.h.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/dmoe.h"
+
+namespace dmoe {
+
+constexpr int kWave = 64;  // CDNA wavefront width
+
+// Thread-local message returned by dmoe_last_error().
+char *error_buffer();
+int fail(int code, const char *fmt, ...);
+
+#define DMOE_REQUIRE(cond, code, ...)            \
+    do {                                         \
+        if (!(cond)) return ::dmoe::fail((code), __VA_ARGS__); \
+    } while (0)
+
+#define DMOE_HIP(expr)                                                              \
+    do {                                                                            \
+        hipError_t err__ = (expr);                                                  \
+        if (err__ != hipSuccess)                                                    \
+            return ::dmoe::fail(DMOE_ERR_HIP, "%s: %s", #expr, hipGetErrorString(err__)); \
+    } while (0)
+
+// Launch errors (bad configuration) surface here; execution stays asynchronous.
+#define DMOE_LAUNCH_CHECK(name)                                                     \
+    do {                                                                            \
+        hipError_t err__ = hipGetLastError();                                       \
+        if (err__ != hipSuccess)                                                    \
+            return ::dmoe::fail(DMOE_ERR_HIP, "launch of %s: %s", (name), hipGetErrorString(err__)); \
+    } while (0)
+
+int device_cus();  // compute units of the current device, cached per device
+
+__device__ __forceinline__ int lane_id() { return threadIdx.x & (kWave - 1); }
+
+// bf16 <-> fp32, round to nearest even (NaN kept quiet).
+__device__ __forceinline__ float bf16_to_f32(uint16_t v) { return __uint_as_float(((uint32_t)v) << 16); }
+__device__ __forceinline__ uint16_t f32_to_bf16(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+    return (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
+}
+
+}  // namespace dmoe

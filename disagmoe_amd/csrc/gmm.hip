@@ -1,0 +1,527 @@
+// Ragged grouped GEMM on CDNA4 matrix cores (bf16 and fp8-e4m3), with an
+// optional fused SiLU(gate)*up epilogue for the gate-up projection.
+//
+// Shape of the kernel
+//   * persistent: one workgroup per compute unit walks a list of
+//     (expert, m-tile, n-tile) work items that every workgroup derives from
+//     batch_sizes on the device (prefix sums kept in LDS), so zero-row experts
+//     cost nothing and no host round trip or scratch table is needed;
+//   * work items are ordered m-fastest inside an n-tile, and consecutive blocks
+//     of items are handed to the workgroups of one XCD (workgroup id % 8), so the
+//     m-tiles that share a weight tile run next to each other on one L2;
+//   * a K-slice of 128 bytes per row (64 bf16 / 128 fp8) of the A and B tiles is
+//     staged global -> registers -> LDS, double buffered; rows are 128 bytes in
+//     LDS with the 16-byte chunk index XOR-swizzled by the row so that both the
+//     MFMA operand reads and the staging writes spread over the banks;
+//   * B in the [E, K, N] layout (N contiguous) is transposed 8x8 in registers on
+//     its way into LDS so that both MFMA operands are read K-contiguous;
+//   * each wavefront owns a TM x TN sub-tile as FM x FN accumulators of
+//     v_mfma_f32_32x32x16_bf16 (v_mfma_f32_32x32x64_f8f6f4 for fp8).
+#include <type_traits>
+
+#include "common.h"
+
+namespace dmoe {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+
+constexpr int kMaxGroups = 1024;   // experts per call (LDS tables)
+constexpr int kRowBytes = 128;     // bytes of K per tile row in LDS
+constexpr int kXcds = 8;
+
+struct GmmArgs {
+    const char *a;
+    const char *b;
+    char *c;
+    const int64_t *batch_sizes;
+    const float *a_scale;
+    const float *b_scale;
+    int64_t rows;   // rows of a / c
+    int E;
+    int K;          // contraction length (elements)
+    int N;          // columns of b per expert (2*I for the swiglu form)
+    int ldc;        // columns of c (N, or I for the swiglu form)
+};
+
+#ifndef DMOE_SWZ_MODE
+#define DMOE_SWZ_MODE 0
+#endif
+// XOR applied to the 16-byte chunk index of a 128-byte LDS row.  Both forms have
+// a period of at most 32 rows, so fragment rows 32 apart differ by a constant.
+__device__ __forceinline__ int swz(int row) { return DMOE_SWZ_MODE == 0 ? (row & 7) : ((row >> 1) & 7); }
+__device__ __forceinline__ int lds_off(int row, int chunk) { return row * kRowBytes + ((chunk ^ swz(row)) << 4); }
+
+template <int BM, int BN, int WM, int WN, bool TRANS_B, bool SWIGLU, bool FP8>
+__global__ __launch_bounds__(WM *WN *kWave) __attribute__((amdgpu_waves_per_eu(WM *WN / 4, WM *WN / 4)))
+void gmm_kernel(const GmmArgs p) {
+    constexpr int NT = WM * WN * kWave;          // threads
+    constexpr int ES = FP8 ? 1 : 2;              // element bytes
+    constexpr int BK = kRowBytes / ES;           // elements of K per tile
+    constexpr int TM = BM / WM, TN = BN / WN;    // wave tile
+    constexpr int FM = TM / 32, FN = TN / 32;    // 32x32 accumulators per wave
+    constexpr int KS = FP8 ? 2 : 4;              // MFMA k-steps per tile
+    constexpr int CA = BM * 8 / NT;              // 16-byte chunks of A per thread per tile
+    constexpr int CB = BN * 8 / NT;
+    constexpr int RSTEP = NT / 8;                // row stride between a thread's chunks
+    constexpr int BNO = SWIGLU ? BN / 2 : BN;    // output columns per tile
+    constexpr int KR = BK * (BN / 8) / NT;       // [E,K,N] layout: k-rows of one 8-column group per thread
+    constexpr int KG = BK / KR;                  // such groups along K
+    constexpr bool FRAG_DB = (WM * WN == 4);     // one wave per SIMD: double-buffer the MFMA operands
+    constexpr int SLOTS = FRAG_DB ? 2 : 1;
+    static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "wave tile");
+    static_assert(CA >= 1 && CB >= 1 && (BM * 8) % NT == 0 && (BN * 8) % NT == 0, "staging split");
+    static_assert(RSTEP % 32 == 0 && (BN / 2) % RSTEP == 0, "staging rows keep their swizzle and their half");
+    static_assert(TRANS_B || ((KR == 8 || KR == 4) && CB == KR), "register transpose handles 8x8 or 4x8 blocks");
+    static_assert(WM * WN % 4 == 0, "whole waves per SIMD");
+    static_assert(!SWIGLU || FN % 2 == 0, "gate and up fragments pair up inside a wave");
+    static_assert(!FP8 || TRANS_B, "fp8 operands are K-contiguous");
+
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    __shared__ int s_tile_start[kMaxGroups + 1];  // m-tiles before expert e
+    __shared__ int s_row_start[kMaxGroups + 1];   // rows before expert e
+    char *sA = smem;                              // [2][BM][128]
+    char *sB = smem + 2 * BM * kRowBytes;         // [2][BN][128]
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = tid / kWave;
+    const int wm = wave / WN, wn = wave % WN;
+    const int E = p.E;
+
+    // ---- work list: prefix sums of rows and m-tiles over the experts ----
+    if (wave == 0) {
+        long long row_carry = 0;
+        int tile_carry = 0;
+        for (int e0 = 0; e0 < E; e0 += kWave) {
+            const int e = e0 + lane;
+            long long n = (e < E) ? (long long)p.batch_sizes[e] : 0;
+            n = n < 0 ? 0 : (n > p.rows ? p.rows : n);
+            long long incl = n;
+#pragma unroll
+            for (int s = 1; s < kWave; s <<= 1) {
+                long long up = __shfl_up(incl, s, kWave);
+                if (lane >= s) incl += up;
+            }
+            long long start = row_carry + incl - n;
+            if (start > p.rows) start = p.rows;
+            long long end = row_carry + incl;
+            if (end > p.rows) end = p.rows;
+            const int mt = (int)((end - start + BM - 1) / BM);
+            int tincl = mt;
+#pragma unroll
+            for (int s = 1; s < kWave; s <<= 1) {
+                int up = __shfl_up(tincl, s, kWave);
+                if (lane >= s) tincl += up;
+            }
+            if (e < E) {
+                s_row_start[e] = (int)start;
+                s_tile_start[e] = tile_carry + tincl - mt;
+            }
+            row_carry += __shfl(incl, kWave - 1, kWave);
+            tile_carry += __shfl(tincl, kWave - 1, kWave);
+        }
+        if (lane == 0) {
+            s_row_start[E] = (int)(row_carry > p.rows ? p.rows : row_carry);
+            s_tile_start[E] = tile_carry;
+        }
+    }
+    __syncthreads();
+
+    const int n_out = SWIGLU ? p.N / 2 : p.N;            // output columns
+    const int n_tiles = (n_out + BNO - 1) / BNO;
+    const int m_tiles = s_tile_start[E];
+    const long long total = (long long)m_tiles * n_tiles;
+    const int KT = (p.K * ES + kRowBytes - 1) / kRowBytes;
+    const int G = gridDim.x;
+    const long long full_rounds = (G % kXcds == 0) ? total / G : 0;  // rounds in which the XCD remap is a bijection
+    const uint32_t a_pitch = (uint32_t)(p.K * ES);       // bytes per row of a (and of b when K-contiguous)
+
+    // per-thread staging coordinates
+    const int a_chunk = tid & 7;
+    const int a_row0 = tid >> 3;
+    const int b_kg = tid % KG;         // [E,K,N] layout: group of KR k-rows ...
+    const int b_ng = tid / KG;         //                 ... of 8 columns
+    const int st_off = lds_off(a_row0, a_chunk);         // rows RSTEP apart share the swizzle
+
+    // per-lane MFMA operand coordinates: row = base + lane % 32, k-group = lane / 32
+    const int l31 = lane & 31;
+    const int kgrp = lane >> 5;
+    const int fa_off = (wm * TM + l31) * kRowBytes;
+    const int fb_off = ((SWIGLU ? wn * (TN / 2) : wn * TN) + l31) * kRowBytes;
+    const int fsw = swz(l31);
+
+    for (long long q = blockIdx.x; q < total; q += G) {
+        // ---- decode the work item ----
+        long long L = q;
+        const long long round = q / G;
+        if (round < full_rounds) {
+            const int w = (int)(q - round * G);
+            L = round * G + (long long)(w % kXcds) * (G / kXcds) + (w / kXcds);
+        }
+        const int u = (int)(L / n_tiles);
+        int lo = 0, hi = E;  // last e with s_tile_start[e] <= u
+        while (hi - lo > 1) {
+            const int mid = (lo + hi) >> 1;
+            if (s_tile_start[mid] <= u) lo = mid; else hi = mid;
+        }
+        const int e = lo;
+        const int mt_e = s_tile_start[e + 1] - s_tile_start[e];
+        const int local = (int)(L - (long long)s_tile_start[e] * n_tiles);
+        const int nt = local / mt_e;
+        const int mi = local - nt * mt_e;
+        const int row0 = s_row_start[e] + mi * BM;             // first row of the tile
+        const int rows_e = s_row_start[e + 1] - row0;          // valid rows from row0 on (>= 1)
+        const int n0 = nt * BNO;                               // first output column
+
+        // ---- staging offsets (bytes from wave-uniform bases) ----
+        const char *a_base = p.a + (long long)row0 * a_pitch;
+        const char *b_exp = p.b + (long long)e * p.K * p.N * ES;
+        // first column of the tile's two halves (plain form: one "half" of BN columns)
+        const char *b_base0, *b_base1;
+        if constexpr (TRANS_B) {
+            b_base0 = b_exp + (long long)n0 * a_pitch;
+            b_base1 = SWIGLU ? b_exp + (long long)(n_out + n0) * a_pitch : b_base0 + (long long)(BN / 2) * a_pitch;
+        } else {
+            b_base0 = b_exp + (long long)n0 * ES;
+            b_base1 = SWIGLU ? b_exp + (long long)(n_out + n0) * ES : b_base0 + (BN / 2) * ES;
+        }
+        const int half_cols = SWIGLU ? n_out - n0 : p.N - n0;  // valid columns from the first column of half 0
+        uint32_t a_off[CA];
+#pragma unroll
+        for (int i = 0; i < CA; ++i) {
+            int r = a_row0 + i * RSTEP;
+            if (r >= rows_e) r = rows_e - 1;                   // clamp: loaded, never stored
+            a_off[i] = (uint32_t)r * a_pitch + a_chunk * 16;
+        }
+        // columns past the end of b are clamped to column 0 of their half: loaded, never stored
+        uint32_t b_off[TRANS_B ? CB : 1];
+        if constexpr (TRANS_B) {
+#pragma unroll
+            for (int i = 0; i < CB; ++i) {
+                const int r = a_row0 + i * RSTEP;              // row of the B tile = output column slot
+                const int rh = (r < BN / 2) ? r : r - BN / 2;  // column inside its half
+                const bool ok = SWIGLU ? rh < half_cols : r < half_cols;
+                b_off[i] = (uint32_t)(ok ? rh : 0) * a_pitch + a_chunk * 16;
+            }
+        } else {
+            const int r = b_ng * 8;                            // first of 8 columns, all in one half
+            const int rh = (r < BN / 2) ? r : r - BN / 2;
+            const bool ok = SWIGLU ? rh < half_cols : r < half_cols;  // N % 8 == 0: valid together
+            b_off[0] = (uint32_t)(ok ? rh : 0) * ES;
+        }
+        const bool b_hi_half = !TRANS_B && (b_ng * 8 >= BN / 2);
+
+        u32x4 ra[CA], rb[CB];
+        // kTail: the tile reaches past K; bytes past the end of a row are read as zero
+        auto load_global = [&](int kt, auto tail_tag) {
+            constexpr bool kTail = decltype(tail_tag)::value;
+            const bool k_ok = !kTail || (kt * kRowBytes + a_chunk * 16 < p.K * ES);
+            const char *ak = a_base + (long long)kt * kRowBytes;
+#pragma unroll
+            for (int i = 0; i < CA; ++i) {
+                if (kTail) ra[i] = u32x4{0, 0, 0, 0};
+                if (k_ok) ra[i] = *(const u32x4 *)(ak + a_off[i]);
+            }
+            if constexpr (TRANS_B) {
+#pragma unroll
+                for (int i = 0; i < CB; ++i) {
+                    const char *bk = ((i * RSTEP < BN / 2) ? b_base0 : b_base1) + (long long)kt * kRowBytes;
+                    if (kTail) rb[i] = u32x4{0, 0, 0, 0};
+                    if (k_ok) rb[i] = *(const u32x4 *)(bk + b_off[i]);
+                }
+            } else {
+                const int k_first = kt * BK + b_kg * KR;
+                const char *bk = (b_hi_half ? b_base1 : b_base0) + (long long)k_first * p.N * ES + b_off[0];
+#pragma unroll
+                for (int j = 0; j < KR; ++j) {
+                    if (kTail) rb[j] = u32x4{0, 0, 0, 0};
+                    if (!kTail || k_first + j < p.K) rb[j] = *(const u32x4 *)(bk + (long long)j * p.N * ES);
+                }
+            }
+        };
+        const int KT_full = (p.K * ES) / kRowBytes;            // tiles that lie inside K entirely
+        auto load_tile = [&](int kt) {
+            if (kt < KT_full) load_global(kt, std::false_type{});
+            else load_global(kt, std::true_type{});
+        };
+        auto store_lds = [&](int buf) {
+            char *dA = sA + buf * BM * kRowBytes + st_off;
+            char *dB = sB + buf * BN * kRowBytes;
+#pragma unroll
+            for (int i = 0; i < CA; ++i) *(u32x4 *)(dA + i * RSTEP * kRowBytes) = ra[i];
+            if constexpr (TRANS_B) {
+#pragma unroll
+                for (int i = 0; i < CB; ++i) *(u32x4 *)(dB + st_off + i * RSTEP * kRowBytes) = rb[i];
+            } else if constexpr (KR == 8) {
+                // rb[j] holds k = j, columns 0..7 (dword c = columns 2c, 2c+1); column n wants k = 0..7
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    u32x4 even, odd;
+#pragma unroll
+                    for (int c2 = 0; c2 < 4; ++c2) {
+                        const uint32_t x = rb[2 * c2][c], y = rb[2 * c2 + 1][c];
+                        even[c2] = (x & 0xffffu) | (y << 16);
+                        odd[c2] = (x >> 16) | (y & 0xffff0000u);
+                    }
+                    *(u32x4 *)(dB + lds_off(b_ng * 8 + 2 * c, b_kg)) = even;
+                    *(u32x4 *)(dB + lds_off(b_ng * 8 + 2 * c + 1, b_kg)) = odd;
+                }
+            } else {
+                // 4 k-rows per thread: each column gets half a chunk (8 bytes)
+                const int half = (b_kg & 1) * 8;
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    uint2 even, odd;
+                    const uint32_t x0 = rb[0][c], y0 = rb[1][c], x1 = rb[2][c], y1 = rb[3][c];
+                    even.x = (x0 & 0xffffu) | (y0 << 16);
+                    even.y = (x1 & 0xffffu) | (y1 << 16);
+                    odd.x = (x0 >> 16) | (y0 & 0xffff0000u);
+                    odd.y = (x1 >> 16) | (y1 & 0xffff0000u);
+                    *(uint2 *)(dB + lds_off(b_ng * 8 + 2 * c, b_kg >> 1) + half) = even;
+                    *(uint2 *)(dB + lds_off(b_ng * 8 + 2 * c + 1, b_kg >> 1) + half) = odd;
+                }
+            }
+        };
+
+        typedef typename std::conditional<FP8, i32x8, bf16x8>::type frag_t;
+        frag_t fa[SLOTS][FM], fb[SLOTS][FN];
+        auto frag_row_b = [&](int j) {  // row offset of B fragment j from fb_off, in rows
+            if (SWIGLU) return (j < FN / 2) ? j * 32 : BN / 2 + (j - FN / 2) * 32;
+            return j * 32;
+        };
+        auto load_frags = [&](int buf, int ks, int slot) {
+            const char *tA = sA + buf * BM * kRowBytes + fa_off;
+            const char *tB = sB + buf * BN * kRowBytes + fb_off;
+            if constexpr (FP8) {
+                const int c0 = ((ks * 4 + kgrp * 2) ^ fsw) << 4, c1 = ((ks * 4 + kgrp * 2 + 1) ^ fsw) << 4;
+#pragma unroll
+                for (int i = 0; i < FM; ++i) {
+                    const u32x4 x0 = *(const u32x4 *)(tA + i * 32 * kRowBytes + c0);
+                    const u32x4 x1 = *(const u32x4 *)(tA + i * 32 * kRowBytes + c1);
+                    const i32x8 v = {(int)x0[0], (int)x0[1], (int)x0[2], (int)x0[3], (int)x1[0], (int)x1[1], (int)x1[2], (int)x1[3]};
+                    fa[slot][i] = v;
+                }
+#pragma unroll
+                for (int j = 0; j < FN; ++j) {
+                    const u32x4 x0 = *(const u32x4 *)(tB + frag_row_b(j) * kRowBytes + c0);
+                    const u32x4 x1 = *(const u32x4 *)(tB + frag_row_b(j) * kRowBytes + c1);
+                    const i32x8 v = {(int)x0[0], (int)x0[1], (int)x0[2], (int)x0[3], (int)x1[0], (int)x1[1], (int)x1[2], (int)x1[3]};
+                    fb[slot][j] = v;
+                }
+            } else {
+                const int c0 = ((ks * 2 + kgrp) ^ fsw) << 4;
+#pragma unroll
+                for (int i = 0; i < FM; ++i) {
+                    const u32x4 x = *(const u32x4 *)(tA + i * 32 * kRowBytes + c0);
+                    __builtin_memcpy(&fa[slot][i], &x, sizeof(x));
+                }
+#pragma unroll
+                for (int j = 0; j < FN; ++j) {
+                    const u32x4 x = *(const u32x4 *)(tB + frag_row_b(j) * kRowBytes + c0);
+                    __builtin_memcpy(&fb[slot][j], &x, sizeof(x));
+                }
+            }
+        };
+        auto mfma_all = [&](f32x16 (&acc)[FM][FN], int slot) {
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+#pragma unroll
+                for (int j = 0; j < FN; ++j) {
+                    if constexpr (FP8)
+                        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[slot][i], fb[slot][j], acc[i][j], 0, 0, 0, 0, 0, 0);
+                    else
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[slot][i], fb[slot][j], acc[i][j], 0, 0, 0);
+                }
+        };
+
+        f32x16 acc[FM][FN];
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+#pragma unroll
+            for (int j = 0; j < FN; ++j)
+#pragma unroll
+                for (int x = 0; x < 16; ++x) acc[i][j][x] = 0.f;
+
+        // ---- prologue ----
+        load_tile(0);
+        store_lds(0);
+        if (KT > 1) load_tile(1);
+        __syncthreads();
+        if constexpr (FRAG_DB) load_frags(0, 0, 0);
+
+        // ---- main loop over K tiles ----
+        for (int kt = 0; kt < KT; ++kt) {
+            const int cur = kt & 1;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                if constexpr (FRAG_DB) {
+                    const int slot = ks & 1;
+                    if (ks + 1 < KS) load_frags(cur, ks + 1, slot ^ 1);
+                    if (ks == KS - 2) {
+                        if (kt + 1 < KT) store_lds(cur ^ 1);
+                        if (kt + 2 < KT) load_tile(kt + 2);
+                    }
+                    if (ks == KS - 1) {
+                        __syncthreads();
+                        if (kt + 1 < KT) load_frags(cur ^ 1, 0, slot ^ 1);
+                    }
+                    mfma_all(acc, slot);
+                } else {
+                    // two waves per SIMD cover each other's LDS latency: operands are read just in time
+                    load_frags(cur, ks, 0);
+                    if (ks == KS - 2) {
+                        if (kt + 1 < KT) store_lds(cur ^ 1);
+                        if (kt + 2 < KT) load_tile(kt + 2);
+                    }
+                    mfma_all(acc, 0);
+                    if (ks == KS - 1) __syncthreads();
+                }
+            }
+        }
+
+        // ---- epilogue: accumulator (row, col) = ((x/4)*8 + (lane/32)*4 + x%4, lane%32) ----
+        uint16_t *cbase = (uint16_t *)p.c;
+        constexpr int FNO = SWIGLU ? FN / 2 : FN;
+#pragma unroll
+        for (int i = 0; i < FM; ++i) {
+#pragma unroll
+            for (int j = 0; j < FNO; ++j) {
+                const int ccol = n0 + (SWIGLU ? wn * (TN / 2) : wn * TN) + j * 32 + l31;
+                if (ccol >= n_out) continue;
+                float sb0 = 1.f, sb1 = 1.f;
+                if (FP8) {
+                    sb0 = p.b_scale[(long long)e * p.N + ccol];
+                    if (SWIGLU) sb1 = p.b_scale[(long long)e * p.N + n_out + ccol];
+                }
+#pragma unroll
+                for (int x = 0; x < 16; ++x) {
+                    const int r = wm * TM + i * 32 + (x >> 2) * 8 + kgrp * 4 + (x & 3);
+                    if (r >= rows_e) continue;
+                    float sa = 1.f;
+                    if (FP8) sa = p.a_scale[row0 + r];
+                    float v;
+                    if (SWIGLU) {
+                        const float g = acc[i][j][x] * (sa * sb0);
+                        const float up = acc[i][j + FN / 2][x] * (sa * sb1);
+                        v = g / (1.f + __expf(-g)) * up;
+                    } else {
+                        v = acc[i][j][x] * (sa * sb0);
+                    }
+                    cbase[(long long)(row0 + r) * p.ldc + ccol] = f32_to_bf16(v);
+                }
+            }
+        }
+    }
+}
+
+template <int BM, int BN, int WM, int WN, bool TRANS_B, bool SWIGLU, bool FP8>
+static int launch_one(const GmmArgs &args, hipStream_t stream) {
+    constexpr int NT = WM * WN * kWave;
+    constexpr int BNO = SWIGLU ? BN / 2 : BN;
+    const size_t lds = 2 * (size_t)(BM + BN) * kRowBytes;
+    auto kern = gmm_kernel<BM, BN, WM, WN, TRANS_B, SWIGLU, FP8>;
+    static bool configured = false;  // the attribute is per function, not per device context switch
+    if (!configured) {
+        DMOE_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        configured = true;
+    }
+    const int n_out = SWIGLU ? args.N / 2 : args.N;
+    const long long n_tiles = (n_out + BNO - 1) / BNO;
+    const long long m_tiles_max = args.rows / BM + args.E;  // sum of ceil(n_e / BM) never exceeds this
+    long long grid = (long long)device_cus();
+    if (m_tiles_max * n_tiles < grid) grid = m_tiles_max * n_tiles;
+    if (grid < 1) grid = 1;
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NT), lds, stream, args);
+    DMOE_LAUNCH_CHECK("gmm_kernel");
+    return DMOE_OK;
+}
+
+static int g_variant = 0;  // 0: 8 wavefronts per 256x256 tile, 1: 4 wavefronts
+
+template <bool TRANS_B, bool SWIGLU, bool FP8>
+static int launch_by_rows(const GmmArgs &args, hipStream_t stream) {
+    // rows per expert on average decide the m-tile; the host does not know the split
+    const long long avg = args.rows / (args.E > 0 ? args.E : 1);
+    if (g_variant == 2) return launch_one<64, 256, 1, 4, TRANS_B, SWIGLU, FP8>(args, stream);
+    if (g_variant == 3) return launch_one<128, 256, 1, 4, TRANS_B, SWIGLU, FP8>(args, stream);
+    if (avg <= 64 && g_variant == 0) return launch_one<64, 256, 1, 4, TRANS_B, SWIGLU, FP8>(args, stream);
+    if (avg <= 160 && g_variant == 0) return launch_one<128, 256, 1, 4, TRANS_B, SWIGLU, FP8>(args, stream);
+    if (g_variant == 1) return launch_one<256, 256, 2, 2, TRANS_B, SWIGLU, FP8>(args, stream);
+    return launch_one<256, 256, 2, 4, TRANS_B, SWIGLU, FP8>(args, stream);
+}
+
+static int check_gmm(const char *who, const void *a, const void *b, const void *c, const int64_t *bs, int64_t rows,
+                     int E, int64_t K, int64_t N, int align) {
+    DMOE_REQUIRE(rows >= 0 && rows < (1ll << 31), DMOE_ERR_SHAPE, "%s: rows=%lld outside [0, 2^31)", who, (long long)rows);
+    DMOE_REQUIRE(E > 0 && E <= kMaxGroups, DMOE_ERR_SHAPE, "%s: E=%d outside [1, %d]", who, E, kMaxGroups);
+    DMOE_REQUIRE(K > 0 && K < (1ll << 22) && K % align == 0, DMOE_ERR_SHAPE, "%s: K=%lld must be a positive multiple of %d",
+                 who, (long long)K, align);
+    DMOE_REQUIRE(N > 0 && N < (1ll << 24) && N % 8 == 0, DMOE_ERR_SHAPE, "%s: N=%lld must be a positive multiple of 8", who,
+                 (long long)N);
+    DMOE_REQUIRE(bs != nullptr && b != nullptr, DMOE_ERR_ARG, "%s: null pointer", who);
+    DMOE_REQUIRE(rows == 0 || (a != nullptr && c != nullptr), DMOE_ERR_ARG, "%s: null pointer", who);
+    return DMOE_OK;
+}
+
+}  // namespace dmoe
+
+using namespace dmoe;
+
+extern "C" int dmoe_gmm_tune(int variant) {
+    DMOE_REQUIRE(variant >= 0 && variant <= 3, DMOE_ERR_ARG, "dmoe_gmm_tune: variant %d outside [0, 3]", variant);
+    g_variant = variant;
+    return DMOE_OK;
+}
+
+extern "C" int dmoe_gmm_workspace_bytes(int E, size_t *bytes) {
+    DMOE_REQUIRE(bytes != nullptr, DMOE_ERR_ARG, "dmoe_gmm_workspace_bytes: null output");
+    DMOE_REQUIRE(E > 0 && E <= kMaxGroups, DMOE_ERR_SHAPE, "dmoe_gmm_workspace_bytes: E=%d outside [1, %d]", E, kMaxGroups);
+    *bytes = 256;  // the work list lives in LDS; a token allocation keeps the reference's calling pattern valid
+    return DMOE_OK;
+}
+
+extern "C" int dmoe_gmm(const void *a, const void *b, void *c, const int64_t *batch_sizes, int64_t rows, int E,
+                        int64_t K, int64_t N, int trans_b, int dtype, void *stream) {
+    DMOE_REQUIRE(dtype == DMOE_BF16, DMOE_ERR_DTYPE, "dmoe_gmm: dtype %d (bf16 only)", dtype);
+    int rc = check_gmm("dmoe_gmm", a, b, c, batch_sizes, rows, E, K, N, 8);
+    if (rc != DMOE_OK) return rc;
+    if (rows == 0) return DMOE_OK;
+    GmmArgs args{(const char *)a, (const char *)b, (char *)c, batch_sizes, nullptr, nullptr, rows, E, (int)K, (int)N, (int)N};
+    return trans_b ? launch_by_rows<true, false, false>(args, (hipStream_t)stream)
+                   : launch_by_rows<false, false, false>(args, (hipStream_t)stream);
+}
+
+extern "C" int dmoe_gmm_swiglu(const void *a, const void *b, void *h, const int64_t *batch_sizes, int64_t rows, int E,
+                               int64_t K, int64_t I, int trans_b, int dtype, void *stream) {
+    DMOE_REQUIRE(dtype == DMOE_BF16, DMOE_ERR_DTYPE, "dmoe_gmm_swiglu: dtype %d (bf16 only)", dtype);
+    int rc = check_gmm("dmoe_gmm_swiglu", a, b, h, batch_sizes, rows, E, K, I, 8);
+    if (rc != DMOE_OK) return rc;
+    if (rows == 0) return DMOE_OK;
+    GmmArgs args{(const char *)a, (const char *)b, (char *)h, batch_sizes, nullptr, nullptr, rows, E, (int)K, (int)(2 * I), (int)I};
+    return trans_b ? launch_by_rows<true, true, false>(args, (hipStream_t)stream)
+                   : launch_by_rows<false, true, false>(args, (hipStream_t)stream);
+}
+
+extern "C" int dmoe_gmm_fp8(const void *a, const float *a_scale, const void *b, const float *b_scale, void *c,
+                            const int64_t *batch_sizes, int64_t rows, int E, int64_t K, int64_t N, void *stream) {
+    int rc = check_gmm("dmoe_gmm_fp8", a, b, c, batch_sizes, rows, E, K, N, 16);
+    if (rc != DMOE_OK) return rc;
+    DMOE_REQUIRE(b_scale != nullptr && (rows == 0 || a_scale != nullptr), DMOE_ERR_ARG, "dmoe_gmm_fp8: null scales");
+    if (rows == 0) return DMOE_OK;
+    GmmArgs args{(const char *)a, (const char *)b, (char *)c, batch_sizes, a_scale, b_scale, rows, E, (int)K, (int)N, (int)N};
+    return launch_by_rows<true, false, true>(args, (hipStream_t)stream);
+}
+
+extern "C" int dmoe_gmm_fp8_swiglu(const void *a, const float *a_scale, const void *b, const float *b_scale, void *h,
+                                   const int64_t *batch_sizes, int64_t rows, int E, int64_t K, int64_t I,
+                                   void *stream) {
+    int rc = check_gmm("dmoe_gmm_fp8_swiglu", a, b, h, batch_sizes, rows, E, K, I, 16);
+    if (rc != DMOE_OK) return rc;
+    DMOE_REQUIRE(b_scale != nullptr && (rows == 0 || a_scale != nullptr), DMOE_ERR_ARG, "dmoe_gmm_fp8_swiglu: null scales");
+    if (rows == 0) return DMOE_OK;
+    GmmArgs args{(const char *)a, (const char *)b, (char *)h, batch_sizes, a_scale, b_scale, rows, E, (int)K, (int)(2 * I), (int)I};
+    return launch_by_rows<true, true, true>(args, (hipStream_t)stream);
+}

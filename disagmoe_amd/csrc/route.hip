@@ -1,0 +1,222 @@
+// Routing: expert ids -> destination rows, per-expert counts and offsets.
+//
+// Counting sort split in chunks of kChunk rows, one wavefront per chunk, so that
+// the order of rows inside an expert is fixed by construction (no atomics decide
+// a position):
+//   pass 1  per-chunk histogram                         -> scratch[chunk][E]
+//   pass 2  every chunk sums the histograms before it (its base rank per
+//           expert) and all of them (counts, offsets), then walks its rows 64 at a
+//           time; a row's rank inside the 64 is the number of lower lanes with
+//           the same id, found with log2(E) wave ballots.
+// With a single chunk the two passes run in one launch.
+#include <stdarg.h>
+#include <string.h>
+
+#include "common.h"
+
+namespace dmoe {
+
+static thread_local char g_err[512] = "";
+char *error_buffer() { return g_err; }
+
+int fail(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int device_cus() {
+    static int cached[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    if (cached[dev] == 0) {
+        int cus = 0;
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+            cus = 256;
+        cached[dev] = cus;
+    }
+    return cached[dev];
+}
+
+constexpr int kChunk = 512;       // rows per wavefront
+constexpr int kMaxExperts = 4096; // 3 int tables of E entries must fit in LDS
+
+template <typename IdT>
+__device__ __forceinline__ int load_id(const IdT *ids, int64_t t, int64_t R, int E) {
+    if (t >= R) return -2;  // past the end
+    long long v = (long long)ids[t];
+    return (v >= 0 && v < E) ? (int)v : -1;  // -1: present but invalid
+}
+
+template <typename IdT>
+__global__ __launch_bounds__(kWave) void route_hist_kernel(const IdT *__restrict__ ids, int64_t R, int E,
+                                                          int *__restrict__ chunk_hist) {
+    extern __shared__ int cnt[];
+    const int lane = threadIdx.x;
+    const int64_t base = (int64_t)blockIdx.x * kChunk;
+    for (int e = lane; e < E; e += kWave) cnt[e] = 0;
+    __syncthreads();
+    for (int i = 0; i < kChunk; i += kWave) {
+        int id = load_id(ids, base + i + lane, R, E);
+        if (id >= 0) atomicAdd(&cnt[id], 1);
+    }
+    __syncthreads();
+    for (int e = lane; e < E; e += kWave) chunk_hist[(int64_t)blockIdx.x * E + e] = cnt[e];
+}
+
+template <typename IdT, typename MapT, bool kSingle>
+__global__ __launch_bounds__(kWave) void route_map_kernel(const IdT *__restrict__ ids, int64_t R, int E, int nchunks,
+                                                         const int *__restrict__ chunk_hist, int order,
+                                                         MapT *__restrict__ mappings,
+                                                         int64_t *__restrict__ batch_sizes,
+                                                         int64_t *__restrict__ offsets) {
+    extern __shared__ int sm[];
+    int *run = sm;           // rows of expert e seen before the current 64
+    int *excl = sm + E;      // first destination row of expert e
+    int *tot = sm + 2 * E;   // rows of expert e
+    const int lane = threadIdx.x;
+    const int chunk = blockIdx.x;
+    const int64_t base = (int64_t)chunk * kChunk;
+
+    if (kSingle) {
+        for (int e = lane; e < E; e += kWave) { tot[e] = 0; run[e] = 0; }
+        __syncthreads();
+        for (int i = 0; i < kChunk; i += kWave) {
+            int id = load_id(ids, base + i + lane, R, E);
+            if (id >= 0) atomicAdd(&tot[id], 1);
+        }
+    } else {
+        for (int e = lane; e < E; e += kWave) {
+            int before = 0, all = 0;
+            for (int c = 0; c < nchunks; ++c) {
+                int v = chunk_hist[(int64_t)c * E + e];
+                all += v;
+                if (c < chunk) before += v;
+            }
+            run[e] = before;
+            tot[e] = all;
+        }
+    }
+    __syncthreads();
+
+    // exclusive scan of tot over experts, 64 at a time
+    int carry = 0;
+    for (int e0 = 0; e0 < E; e0 += kWave) {
+        int e = e0 + lane;
+        int v = (e < E) ? tot[e] : 0;
+        int incl = v;
+#pragma unroll
+        for (int s = 1; s < kWave; s <<= 1) {
+            int up = __shfl_up(incl, s, kWave);
+            if (lane >= s) incl += up;
+        }
+        if (e < E) excl[e] = carry + incl - v;
+        carry += __shfl(incl, kWave - 1, kWave);
+    }
+    __syncthreads();
+
+    if (chunk == 0) {
+        for (int e = lane; e < E; e += kWave) {
+            if (batch_sizes) batch_sizes[e] = tot[e];
+            if (offsets) offsets[e] = excl[e];
+        }
+        if (offsets && lane == 0) offsets[E] = carry;
+    }
+
+    int nbits = 0;
+    while ((1 << nbits) < E) ++nbits;
+    const unsigned long long below = (lane == 0) ? 0ull : (~0ull >> (kWave - lane));
+
+    for (int i = 0; i < kChunk; i += kWave) {
+        const int64_t t = base + i + lane;
+        const int id = load_id(ids, t, R, E);
+        const bool ok = id >= 0;
+        unsigned long long same = __ballot(ok);
+        for (int b = 0; b < nbits; ++b) {
+            const bool bit = ok && ((id >> b) & 1);
+            const unsigned long long bal = __ballot(bit);
+            same &= bit ? bal : ~bal;
+        }
+        const int lower = __popcll(same & below);
+        const int total = __popcll(same);
+        const int seen = ok ? run[id] : 0;
+        __syncthreads();
+        if (ok && lower == 0) run[id] = seen + total;
+        __syncthreads();
+        if (ok) {
+            const int rank = seen + lower;
+            const int pos = (order == DMOE_ORDER_REFERENCE) ? excl[id] + tot[id] - 1 - rank : excl[id] + rank;
+            mappings[t] = (MapT)pos;
+        } else if (id == -1) {
+            mappings[t] = (MapT)-1;
+        }
+    }
+}
+
+template <typename IdT, typename MapT>
+static int launch_route(const void *ids, int64_t R, int E, int order, void *mappings, int64_t *batch_sizes,
+                        int64_t *offsets, void *scratch, hipStream_t stream) {
+    const int nchunks = (int)((R + kChunk - 1) / kChunk);
+    const size_t lds = 3 * (size_t)E * sizeof(int);
+    if (nchunks <= 1) {
+        hipLaunchKernelGGL((route_map_kernel<IdT, MapT, true>), dim3(1), dim3(kWave), lds, stream, (const IdT *)ids, R,
+                           E, 1, (const int *)nullptr, order, (MapT *)mappings, batch_sizes, offsets);
+        DMOE_LAUNCH_CHECK("route_map_kernel");
+        return DMOE_OK;
+    }
+    hipLaunchKernelGGL((route_hist_kernel<IdT>), dim3(nchunks), dim3(kWave), (size_t)E * sizeof(int), stream,
+                       (const IdT *)ids, R, E, (int *)scratch);
+    DMOE_LAUNCH_CHECK("route_hist_kernel");
+    hipLaunchKernelGGL((route_map_kernel<IdT, MapT, false>), dim3(nchunks), dim3(kWave), lds, stream,
+                       (const IdT *)ids, R, E, nchunks, (const int *)scratch, order, (MapT *)mappings, batch_sizes,
+                       offsets);
+    DMOE_LAUNCH_CHECK("route_map_kernel");
+    return DMOE_OK;
+}
+
+}  // namespace dmoe
+
+using namespace dmoe;
+
+extern "C" const char *dmoe_version(void) { return "dmoe-hip gfx950 0.1"; }
+extern "C" const char *dmoe_last_error(void) { return error_buffer(); }
+
+extern "C" int dmoe_device_cus(int *cus) {
+    DMOE_REQUIRE(cus != nullptr, DMOE_ERR_ARG, "dmoe_device_cus: null output");
+    *cus = device_cus();
+    return DMOE_OK;
+}
+
+extern "C" int dmoe_route_scratch_bytes(int64_t R, int E, size_t *bytes) {
+    DMOE_REQUIRE(bytes != nullptr, DMOE_ERR_ARG, "dmoe_route_scratch_bytes: null output");
+    DMOE_REQUIRE(R >= 0 && R < (1ll << 31), DMOE_ERR_SHAPE, "dmoe_route: R=%lld outside [0, 2^31)", (long long)R);
+    DMOE_REQUIRE(E > 0 && E <= kMaxExperts, DMOE_ERR_SHAPE, "dmoe_route: E=%d outside [1, %d]", E, kMaxExperts);
+    const int64_t nchunks = (R + kChunk - 1) / kChunk;
+    *bytes = (nchunks <= 1) ? 0 : (size_t)nchunks * (size_t)E * sizeof(int);
+    return DMOE_OK;
+}
+
+extern "C" int dmoe_route(const void *ids, int ids_type, int64_t R, int E, int order, void *mappings, int map_type,
+                          int64_t *batch_sizes, int64_t *offsets, void *scratch, size_t scratch_bytes,
+                          void *stream) {
+    size_t need = 0;
+    int rc = dmoe_route_scratch_bytes(R, E, &need);
+    if (rc != DMOE_OK) return rc;
+    DMOE_REQUIRE(order == DMOE_ORDER_REFERENCE || order == DMOE_ORDER_STABLE, DMOE_ERR_ARG,
+                 "dmoe_route: unknown order %d", order);
+    DMOE_REQUIRE(ids_type == DMOE_I32 || ids_type == DMOE_I64, DMOE_ERR_DTYPE, "dmoe_route: ids type %d", ids_type);
+    DMOE_REQUIRE(map_type == DMOE_I32 || map_type == DMOE_I64, DMOE_ERR_DTYPE, "dmoe_route: mapping type %d",
+                 map_type);
+    DMOE_REQUIRE(R == 0 || (ids != nullptr && mappings != nullptr), DMOE_ERR_ARG, "dmoe_route: null ids/mappings");
+    DMOE_REQUIRE(need == 0 || (scratch != nullptr && scratch_bytes >= need), DMOE_ERR_WORKSPACE,
+                 "dmoe_route: scratch of %zu bytes needed, %zu given", need, scratch_bytes);
+    hipStream_t s = (hipStream_t)stream;
+    if (ids_type == DMOE_I32) {
+        if (map_type == DMOE_I32) return launch_route<int32_t, int32_t>(ids, R, E, order, mappings, batch_sizes, offsets, scratch, s);
+        return launch_route<int32_t, int64_t>(ids, R, E, order, mappings, batch_sizes, offsets, scratch, s);
+    }
+    if (map_type == DMOE_I32) return launch_route<int64_t, int32_t>(ids, R, E, order, mappings, batch_sizes, offsets, scratch, s);
+    return launch_route<int64_t, int64_t>(ids, R, E, order, mappings, batch_sizes, offsets, scratch, s);
+}

@@ -1,0 +1,130 @@
+"""Expert layer modules with the constructor, parameters and ``forward`` of the
+reference's ``disagmoe/models/experts.py`` (MoEExperts :9-96, MoEExpertsSerial
+:98-120), running on the HIP grouped GEMM.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from ..grouped_gemm import backend as gg
+
+MAX_BATCH_SIZE = 256  # disagmoe/utils/constants.py:20-22
+
+
+class MoEExperts(torch.nn.Module):
+    """Fused-w13 SwiGLU experts.
+
+    Parameters (experts.py:42-55): ``w13_weight [E, d, 2I]`` (gate = columns
+    ``[0, I)``, up = ``[I, 2I)``) and ``w2_weight [E, I, d]``, bf16, no grad.
+    ``forward(bs, hiddens, batch_sizes)`` (:81-96) maps expert-sorted rows
+    ``[R, d]`` to ``[R, d]``.
+    """
+
+    def __init__(self, hidden_size: int, intermediate_size: int, num_experts: int, tp_size: int = 1,
+                 enable_cutlass_cache: bool = True, max_batch_size: int = MAX_BATCH_SIZE,
+                 device: Optional[torch.device] = None, init_std: float = 1.0):
+        super().__init__()
+        self.hidden_size = hidden_size
+        self.intermediate_size = intermediate_size
+        self.num_experts = num_experts
+        self.tp_size = tp_size
+        assert tp_size == 1, "Not implemented TP for experts yet"  # experts.py:24
+        self._device = torch.device(device) if device is not None else torch.device("cuda", torch.cuda.current_device())
+        self._init_std = init_std
+        self.create_weights(enable_cutlass_cache=enable_cutlass_cache, max_batch_size=max_batch_size)
+        self.gmm = gg.gmm
+        self.gmm_cache_max_batch_size = max_batch_size
+
+    def create_weights(self, params_dtype: Optional[torch.dtype] = None, enable_cutlass_cache: bool = False,
+                       max_batch_size: int = MAX_BATCH_SIZE):
+        params_dtype = params_dtype or torch.bfloat16
+        dev = self._device
+
+        def randn(*shape):
+            # generated on the device expert by expert: the full fp32 tensor never exists
+            w = torch.empty(shape, dtype=params_dtype, device=dev)
+            for e in range(shape[0]):
+                w[e] = (torch.randn(shape[1:], dtype=torch.float32, device=dev) * self._init_std).to(params_dtype)
+            return w
+
+        self.w13_weight = torch.nn.Parameter(randn(self.num_experts, self.hidden_size, self.intermediate_size * 2),
+                                             requires_grad=False)
+        self.w2_weight = torch.nn.Parameter(randn(self.num_experts, self.intermediate_size, self.hidden_size),
+                                            requires_grad=False)
+        self.act_fn = torch.nn.SiLU(inplace=True)
+        # static buffers for batches below max_batch_size (experts.py:66-67): forward does not allocate
+        self.cache_up = torch.empty((max_batch_size, self.intermediate_size), dtype=params_dtype, device=dev)
+        self.cache_down = torch.empty((max_batch_size, self.hidden_size), dtype=params_dtype, device=dev)
+        self.enable_cache = enable_cutlass_cache
+        if enable_cutlass_cache:
+            self.workspace_size, self.arguments_ptr = gg.get_arguments(self.num_experts, dev)
+            self.workspace = torch.empty([self.workspace_size], dtype=torch.uint8, device=dev)
+
+    def forward(self, bs: int, hiddens: torch.Tensor, batch_sizes: torch.Tensor) -> torch.Tensor:
+        """``gmm(silu(u[:, :I]) * u[:, I:], w2)`` with ``u = gmm(hiddens, w13)``
+        (experts.py:92-96); gate-up, SiLU and the product are one kernel.  Below
+        ``max_batch_size`` rows the static buffers are used (the reference's
+        cached branch, :83-90)."""
+        if self.enable_cache and bs <= self.gmm_cache_max_batch_size and hiddens.shape[0] <= self.cache_up.shape[0]:
+            h = gg.gmm_swiglu(hiddens, self.w13_weight, batch_sizes, c=self.cache_up)[:hiddens.shape[0]]
+            return gg.gmm(h, self.w2_weight, batch_sizes, c=self.cache_down)[:hiddens.shape[0]]
+        h = gg.gmm_swiglu(hiddens, self.w13_weight, batch_sizes)
+        return gg.gmm(h, self.w2_weight, batch_sizes)
+
+    def forward_unfused(self, bs: int, hiddens: torch.Tensor, batch_sizes: torch.Tensor) -> torch.Tensor:
+        """The reference's own schedule, statement by statement (experts.py:92-94):
+        the gate-up result, SiLU and the product are each rounded to bf16."""
+        up = self.gmm(hiddens, self.w13_weight, batch_sizes)
+        up = self.act_fn(up[:, :self.intermediate_size]) * up[:, self.intermediate_size:]
+        return self.gmm(up, self.w2_weight, batch_sizes)
+
+
+class MoEExpertsSerial(MoEExperts):
+    """Per-expert loop of plain library matmuls (experts.py:98-120; selected by
+    ``enable_grouped_gemm=False``, executor.py:353).  The reference reads
+    ``w1_weight``/``w3_weight`` that it never creates; here they are the two
+    halves of ``w13_weight`` as the layout comment (:42-47) defines them.  Reads
+    ``batch_sizes`` on the host (one synchronisation), like the reference's loop."""
+
+    def __init__(self, hidden_size, intermediate_size, num_experts, tp_size=1, max_batch_size: int = MAX_BATCH_SIZE,
+                 **kwargs):
+        super().__init__(hidden_size, intermediate_size, num_experts, tp_size, enable_cutlass_cache=False,
+                         max_batch_size=max_batch_size, **kwargs)
+
+    def forward(self, num_tokens: int, hiddens: torch.Tensor, batch_sizes: torch.Tensor) -> torch.Tensor:
+        inter = self.intermediate_size
+        results = []
+        s = 0
+        single = batch_sizes.shape[0] == 1
+        for i, n in enumerate(batch_sizes.tolist()):
+            cur = hiddens if single else hiddens[s:s + n]
+            gate = torch.matmul(cur, self.w13_weight[i, :, :inter])
+            up = torch.matmul(cur, self.w13_weight[i, :, inter:])
+            results.append(torch.matmul(self.act_fn(gate) * up, self.w2_weight[i]))
+            s += n
+        return torch.cat(results)
+
+
+class MoEExpertsFP8(torch.nn.Module):
+    """fp8-e4m3 experts (no counterpart in the reference): weights quantised per
+    output channel and stored K-contiguous (``w13_q [E, 2I, d]``, ``w2_q [E, d,
+    I]``), activations quantised per row on the fly, bf16 in and out."""
+
+    def __init__(self, w13: torch.Tensor, w2: torch.Tensor):
+        super().__init__()
+        self.num_experts, self.hidden_size, two_i = w13.shape
+        self.intermediate_size = two_i // 2
+        q13, s13 = gg.quantize_weight(w13)
+        q2, s2 = gg.quantize_weight(w2)
+        self.w13_q = torch.nn.Parameter(q13, requires_grad=False)
+        self.w13_scale = torch.nn.Parameter(s13, requires_grad=False)
+        self.w2_q = torch.nn.Parameter(q2, requires_grad=False)
+        self.w2_scale = torch.nn.Parameter(s2, requires_grad=False)
+
+    def forward(self, bs: int, hiddens: torch.Tensor, batch_sizes: torch.Tensor) -> torch.Tensor:
+        xq, xs = gg.quantize_rows(hiddens)
+        h = gg.gmm_fp8_swiglu(xq, xs, self.w13_q, self.w13_scale, batch_sizes)
+        hq, hs = gg.quantize_rows(h)
+        return gg.gmm_fp8(hq, hs, self.w2_q, self.w2_scale, batch_sizes)

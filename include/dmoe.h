@@ -1,0 +1,168 @@
+/*
+ * dmoe.h -- C ABI of libdmoe_hip.so: the MI355X (gfx950) expert-worker hot path.
+ *
+ * Routing ids -> expert-sorted row mapping, token permute / gather, ragged
+ * grouped GEMM (bf16 and fp8-e4m3, SiLU*mul fused for the gate-up projection)
+ * and the gate-weighted combine back to token order.
+ *
+ * Conventions for every entry point
+ *   - all data pointers are DEVICE pointers on the current HIP device unless a
+ *     parameter says "host";
+ *   - `stream` is a hipStream_t passed as void*; work is only enqueued, no entry
+ *     point synchronises the device or allocates device memory;
+ *   - the return value is DMOE_OK (0) or a negative DMOE_ERR_* code; nothing
+ *     aborts the process (the reference's CUDACHECK prints and exits,
+ *     csrc/include/cuda_utils.h:22-41, and its shape checks are C asserts,
+ *     csrc/cuda_ops/permute.cu:70,91-98); dmoe_last_error() returns a
+ *     thread-local message for the last failure;
+ *   - tensors are row-major and contiguous (row stride == row length), as the
+ *     reference requires (disagmoe/ops/memory.py:77).
+ */
+#ifndef DMOE_H_
+#define DMOE_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DMOE_OK 0
+#define DMOE_ERR_ARG (-1)       /* null pointer, negative size, bad enum */
+#define DMOE_ERR_SHAPE (-2)     /* shape constraint violated */
+#define DMOE_ERR_DTYPE (-3)     /* unsupported element / index type */
+#define DMOE_ERR_WORKSPACE (-4) /* scratch buffer missing or too small */
+#define DMOE_ERR_HIP (-5)       /* a HIP runtime call failed */
+
+/* element types of row data */
+#define DMOE_BF16 0
+#define DMOE_FP16 1
+#define DMOE_FP8_E4M3 2 /* OCP e4m3fn, max 448 */
+
+/* integer types of ids / mappings: the size in bytes */
+#define DMOE_I32 4
+#define DMOE_I64 8
+
+/* order of rows inside one expert's range (dmoe_route) */
+#define DMOE_ORDER_REFERENCE 0 /* descending t: disagmoe/ops/memory.py:50-52 */
+#define DMOE_ORDER_STABLE 1    /* ascending t: disagmoe/ops/memory.py:57-69 with a stable sort */
+
+/* rounding schedule of dmoe_combine */
+#define DMOE_COMBINE_FP32 0      /* fp32 accumulate, one rounding */
+#define DMOE_COMBINE_REFERENCE 1 /* bf16(w)*y rounded, then left-to-right rounded adds:
+                                    disagmoe/frontend/engine.py:726,732,627 */
+
+const char *dmoe_version(void);
+const char *dmoe_last_error(void);
+
+/* Number of compute units of the current device (persistent-grid size). */
+int dmoe_device_cus(int *cus);
+
+/* ---- routing ------------------------------------------------------------
+ * Replaces the host counting sort get_mappings_from_exp_ids
+ * (disagmoe/ops/memory.py:34-54), its device variant (:57-69), the merge-side
+ * sort Metadata::merge_by_exp_ids (csrc/include/datatypes.hpp:288-337) and the
+ * histogram upload Metadata::get_expert_batch_sizes_cuda (:228-247).
+ *
+ *   ids          [R]   expert id of routed row t (token-major t = i*k + j)
+ *   mappings     [R]   destination row of t in the expert-sorted buffer;
+ *                      -1 for an id outside [0, E)
+ *   batch_sizes  [E]   int64 rows per expert            (may be NULL)
+ *   offsets      [E+1] int64 exclusive scan of the above (may be NULL)
+ *   scratch            dmoe_route_scratch_bytes(R, E) bytes, contents ignored
+ */
+int dmoe_route_scratch_bytes(int64_t R, int E, size_t *bytes);
+int dmoe_route(const void *ids, int ids_type, int64_t R, int E, int order,
+               void *mappings, int map_type, int64_t *batch_sizes, int64_t *offsets,
+               void *scratch, size_t scratch_bytes, void *stream);
+
+/* ---- row movement -------------------------------------------------------
+ * dmoe_permute replaces permute_tokens_cuda(tokens, mappings, stream)
+ * (csrc/include/permute.h:8, csrc/cuda_ops/permute.cu:86-112, bound at
+ * csrc/bindings.cpp:173) and the Triton permute (disagmoe/ops/memory.py:72-91):
+ *     out[mappings[t], :] = in[t / k, :],  k = R / T,  R % T == 0.
+ * Rows whose mapping is outside [0, R) are skipped.  The reference's
+ * d % 2048 == 0 limit (permute.cu:70) is relaxed to row_bytes % 16 == 0.
+ * `row_scale` (optional, [R], same element type as the rows, NULL for none)
+ * multiplies row t before it is stored: the `output * topk_weights` step of
+ * disagmoe/frontend/engine.py:731-732 fused into the return permute.
+ */
+int dmoe_permute(const void *in, void *out, const void *mappings, int map_type,
+                 int64_t T, int64_t R, int64_t d, int dtype, const void *row_scale, void *stream);
+
+/* out[t, :] = in[index[t], :] for t in [0, N); rows with an index outside
+ * [0, n_src) are zero-filled.  Index form of gather_tokens_cuda
+ * (csrc/include/permute.h:10, csrc/cuda_ops/permute.cu:144-152) and of the
+ * torch.index_select permute (tests/dp/test_split.py:33). */
+int dmoe_gather_rows(const void *in, void *out, const void *index, int idx_type,
+                     int64_t N, int64_t n_src, int64_t d, int dtype, void *stream);
+
+/* out[t, :] = *(row*)src_rows[t]: gather_tokens_cuda with the table of raw row
+ * pointers ALREADY on the device (the reference uploads it and synchronises
+ * per call, permute.cu:147,151).  NULL entries are zero-filled. */
+int dmoe_gather_ptrs(const void *const *src_rows, void *out, int64_t N, int64_t d, int dtype,
+                     void *stream);
+
+/* Gate-weighted unpermute back to token order:
+ *     out[i, :] = sum_j w[i, j] * y[mappings[i*k + j], :]
+ * Replaces scale (engine.py:731-732) + return permute (:734) + top-k sum
+ * (:624-628).  `weights` is fp32 [T, k].  Rows with a mapping outside [0, R)
+ * contribute nothing. */
+int dmoe_combine(const void *y, const void *mappings, int map_type, const float *weights,
+                 void *out, int64_t T, int k, int64_t d, int dtype, int mode, void *stream);
+
+/* ---- grouped GEMM -------------------------------------------------------
+ * dmoe_gmm replaces grouped_gemm.backend.gmm(a, b, batch_sizes, trans_b, c)
+ * (third-party; call sites disagmoe/models/experts.py:84,89,92,94 and
+ * tests/ops/test_gemm.py:15):
+ *     c[o_e:o_e+n_e, :] = a[o_e:o_e+n_e, :] @ (trans_b ? b[e]^T : b[e])
+ *   a [rows, K]; b [E, K, N] (or [E, N, K] with trans_b); c [rows, N];
+ *   batch_sizes int64 [E] on the DEVICE; rows past sum(batch_sizes) untouched,
+ *   sizes are clamped so that no row >= `rows` is ever read or written.
+ *   dtype DMOE_BF16: bf16 operands, fp32 accumulate, bf16 result.
+ *   K % 8 == 0 and N % 8 == 0 (16-byte rows).
+ *
+ * dmoe_gmm_swiglu is the gate-up projection of MoEExperts.forward
+ * (experts.py:92-93) with the activation fused:
+ *     h[r, n] = silu(u[r, n]) * u[r, I + n],  u = a @ b[e],  b [E, K, 2I]
+ *   (or [E, 2I, K] with trans_b), h [rows, I]; silu and the product are taken on
+ *   the fp32 accumulators, one rounding.
+ */
+int dmoe_gmm(const void *a, const void *b, void *c, const int64_t *batch_sizes,
+             int64_t rows, int E, int64_t K, int64_t N, int trans_b, int dtype, void *stream);
+int dmoe_gmm_swiglu(const void *a, const void *b, void *h, const int64_t *batch_sizes,
+                    int64_t rows, int E, int64_t K, int64_t I, int trans_b, int dtype, void *stream);
+
+/* Scratch a caller may pre-allocate per the reference's get_arguments()
+ * (experts.py:69-72).  The HIP scheduler derives its tile table from
+ * batch_sizes on the device, so the size is a small constant. */
+int dmoe_gmm_workspace_bytes(int E, size_t *bytes);
+
+/* Tuning hook for benchmarks (no counterpart in the reference): 0 = choose the
+ * tile shape from rows per expert (default); 1 = 256x256 tile on 4 wavefronts;
+ * 2 = 64x256; 3 = 128x256.  Process-wide, not thread-safe. */
+int dmoe_gmm_tune(int variant);
+
+/* ---- fp8 (e4m3) path: no counterpart in the reference ---------------------
+ * Per-row quantisation: q[r, :] = fp8(x[r, :] / s[r]), s[r] = absmax(x[r, :]) / 448
+ * (s = 1 for a zero row).  x is bf16 [rows, d]. */
+int dmoe_quant_rows(const void *x, void *q, float *scales, int64_t rows, int64_t d, int dtype,
+                    void *stream);
+
+/* fp8 grouped GEMM, operands K-contiguous:
+ *   a  fp8 [rows, K] with a_scale fp32 [rows]
+ *   b  fp8 [E, N, K] with b_scale fp32 [E, N]     (per output channel)
+ *   c  bf16 [rows, N] = (a @ b[e]^T) * a_scale[r] * b_scale[e, n]
+ * K % 16 == 0.  The swiglu form takes b [E, 2I, K], b_scale [E, 2I] and writes
+ * h bf16 [rows, I] as dmoe_gmm_swiglu does. */
+int dmoe_gmm_fp8(const void *a, const float *a_scale, const void *b, const float *b_scale, void *c,
+                 const int64_t *batch_sizes, int64_t rows, int E, int64_t K, int64_t N, void *stream);
+int dmoe_gmm_fp8_swiglu(const void *a, const float *a_scale, const void *b, const float *b_scale,
+                        void *h, const int64_t *batch_sizes, int64_t rows, int E, int64_t K,
+                        int64_t I, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DMOE_H_ */

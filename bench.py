@@ -1,0 +1,200 @@
+"""Expert-layer benchmark on one MI355X.
+
+``python bench.py [--gpus 1] [--steps K] [--warmup W] [--config C2]`` times K
+passes of route -> permute -> SwiGLU FFN (grouped GEMM) -> combine over one
+synthetic batch that is already resident in HBM, and prints ONE JSON line:
+tokens/s of the whole step, the roofline record of the dominant kernel (the
+gate-up grouped GEMM) measured with HIP events on the launch stream, the other
+stages' rates, and the CPU path timed on the host cores on a bounded sample.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+# MI355X published peaks
+PEAK_HBM_GBS = 8000.0
+PEAK_BF16_TFLOPS = 2500.0
+PEAK_FP8_TFLOPS = 5000.0
+
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc runs
+# (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known size); None until measured.
+MEASURED_TRAFFIC = {}
+
+
+def _event_ms(fn, iters: int, warmup: int = 2):
+    """Average duration of ``fn`` in ms, HIP events on the current stream (the one
+    the kernels are launched on)."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    start = [torch.cuda.Event(enable_timing=True) for _ in range(iters)]
+    stop = [torch.cuda.Event(enable_timing=True) for _ in range(iters)]
+    for i in range(iters):
+        start[i].record()
+        fn()
+        stop[i].record()
+    torch.cuda.synchronize()
+    times = [s.elapsed_time(e) for s, e in zip(start, stop)]
+    return sum(times) / len(times), min(times)
+
+
+def _cpu_baseline(w, x, ids, gates, layer, budget_s: float = 12.0):
+    """The CPU path (oracle/cpu_path.py) on a growing prefix of the batch until
+    about ``budget_s`` seconds are spent; returns the record of the largest sample."""
+    import torch
+    from oracle import cpu_path
+    cores = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(cores)
+    w13 = layer.w13_weight.detach().cpu()
+    w2 = layer.w2_weight.detach().cpu()
+    xc, idc, gc = x.cpu(), ids.cpu(), gates.cpu()
+    n = min(w.T, 64)
+    spent = 0.0
+    best = None
+    while True:
+        t0 = time.perf_counter()
+        cpu_path.expert_layer(xc[:n], idc[:n], gc[:n], w13, w2)
+        dt = time.perf_counter() - t0
+        spent += dt
+        best = (n, dt)
+        if n >= w.T or spent + 2.2 * dt > budget_s:
+            break
+        n = min(w.T, n * 2)
+    n, dt = best
+    return {"value": n / dt, "unit": "tokens/s", "cores": cores, "kind": "port",
+            "sample": f"first {n} of {w.T} tokens ({n * w.k} routed rows) through all {w.E} experts' full weights, "
+                      f"one pass, {dt:.2f} s; bf16 storage, torch CPU matmul (fp32 accumulate)"}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--config", default="C2", choices=["C1", "C2", "C3", "C4", "C5"])
+    ap.add_argument("--variant", type=int, default=0, help="grouped GEMM tile variant (tuning)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--kernel-iters", type=int, default=10)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: the expert-worker path is built and measured on a single MI355X; "
+              "run with --gpus 1", file=sys.stderr)
+        return 2
+
+    import torch
+    from disagmoe_amd import _lib, workloads
+    from disagmoe_amd.grouped_gemm import backend as gg
+    from disagmoe_amd.models.experts import MoEExperts, MoEExpertsFP8
+    from disagmoe_amd.ops import memory
+
+    assert torch.cuda.is_available(), "bench.py needs a HIP device"
+    _lib.load()
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    w = workloads.WORKLOADS[args.config]
+    gg.set_tile_variant(args.variant)
+
+    ids_cpu, gates_cpu = workloads.make_routing(w)
+    x = workloads.make_activations(w).to(dev)
+    ids, gates = ids_cpu.to(dev), gates_cpu.to(dev)
+    w13, w2 = workloads.make_weights(w, dev)
+    if w.fp8:
+        layer = MoEExpertsFP8(w13, w2)
+        bf16_layer = None
+    else:
+        layer = MoEExperts.__new__(MoEExperts)
+        torch.nn.Module.__init__(layer)
+        layer.hidden_size, layer.intermediate_size, layer.num_experts, layer.tp_size = w.d, w.I, w.E, 1
+        layer.w13_weight = torch.nn.Parameter(w13, requires_grad=False)
+        layer.w2_weight = torch.nn.Parameter(w2, requires_grad=False)
+        layer.enable_cache = False
+        layer.gmm_cache_max_batch_size = 0
+    torch.cuda.synchronize()
+
+    def step():
+        mappings, batch_sizes, _ = memory.route_tokens(ids, w.E)
+        permuted = memory.permute_tokens_cuda(x, mappings)
+        y = layer.forward(w.R, permuted, batch_sizes)
+        return memory.combine_tokens(y, mappings, gates)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+
+    # ---- per-kernel timing (HIP events on the launch stream) ----
+    mappings, batch_sizes, _ = memory.route_tokens(ids, w.E)
+    permuted = memory.permute_tokens_cuda(x, mappings)
+    it = args.kernel_iters
+    stages = {}
+    ms, _ = _event_ms(lambda: memory.route_tokens(ids, w.E), it)
+    stages["route"] = {"ms": ms, "GB/s": w.route_bytes / ms / 1e6}
+    ms, _ = _event_ms(lambda: memory.permute_tokens_cuda(x, mappings), it)
+    stages["permute"] = {"ms": ms, "GB/s": w.permute_bytes / ms / 1e6, "frac_hbm": w.permute_bytes / ms / 1e6 / PEAK_HBM_GBS}
+    if w.fp8:
+        xq, xs = gg.quantize_rows(permuted)
+        h = gg.gmm_fp8_swiglu(xq, xs, layer.w13_q, layer.w13_scale, batch_sizes)
+        hq, hs = gg.quantize_rows(h)
+        up_ms, _ = _event_ms(lambda: gg.gmm_fp8_swiglu(xq, xs, layer.w13_q, layer.w13_scale, batch_sizes, c=h), it)
+        down_ms, _ = _event_ms(lambda: gg.gmm_fp8(hq, hs, layer.w2_q, layer.w2_scale, batch_sizes), it)
+        q_ms, _ = _event_ms(lambda: gg.quantize_rows(permuted), it)
+        stages["quant_rows"] = {"ms": q_ms}
+        peak = PEAK_FP8_TFLOPS
+        kernel = "gmm_kernel<fp8, swiglu> (gate-up)"
+    else:
+        h = gg.gmm_swiglu(permuted, layer.w13_weight, batch_sizes)
+        up_ms, _ = _event_ms(lambda: gg.gmm_swiglu(permuted, layer.w13_weight, batch_sizes, c=h), it)
+        y_buf = torch.empty((w.R, w.d), dtype=torch.bfloat16, device=dev)
+        down_ms, _ = _event_ms(lambda: gg.gmm(h, layer.w2_weight, batch_sizes, c=y_buf), it)
+        peak = PEAK_BF16_TFLOPS
+        kernel = "gmm_kernel<bf16, swiglu> (gate-up)"
+    up_flops = 2.0 * w.R * w.d * 2 * w.I
+    down_flops = 2.0 * w.R * w.I * w.d
+    stages["gemm_gate_up"] = {"ms": up_ms, "TFLOP/s": up_flops / up_ms / 1e9, "frac_mfma": up_flops / up_ms / 1e9 / peak}
+    stages["gemm_down"] = {"ms": down_ms, "TFLOP/s": down_flops / down_ms / 1e9, "frac_mfma": down_flops / down_ms / 1e9 / peak}
+    stages["gemm_total"] = {"ms": up_ms + down_ms, "TFLOP/s": w.gemm_flops / (up_ms + down_ms) / 1e9,
+                            "frac_mfma": w.gemm_flops / (up_ms + down_ms) / 1e9 / peak}
+    y = layer.forward(w.R, permuted, batch_sizes)
+    ms, _ = _event_ms(lambda: memory.combine_tokens(y, mappings, gates), it)
+    stages["combine"] = {"ms": ms, "GB/s": w.combine_bytes / ms / 1e6, "frac_hbm": w.combine_bytes / ms / 1e6 / PEAK_HBM_GBS}
+
+    achieved = up_flops / up_ms / 1e9
+    roofline = {"kernel": kernel, "bound": "mfma", "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
+                "frac": achieved / peak, "traffic": MEASURED_TRAFFIC.get(args.config),
+                "flops_per_launch": up_flops, "avg_launch_ms": up_ms}
+
+    record = {
+        "metric": "expert-layer tokens/s (route + permute + grouped-GEMM SwiGLU FFN + combine)",
+        "value": w.T / (ms_per_step / 1e3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "fp8_e4m3" if w.fp8 else "bf16", "data": "synthetic",
+        "config": {"workload": w.name, "E": w.E, "d": w.d, "ffn": w.I, "T": w.T, "top_k": w.k,
+                   "routed_rows": w.R, "routing": w.routing, "tile_variant": args.variant},
+        "roofline": roofline,
+        "stages": {k: {kk: (round(vv, 5) if isinstance(vv, float) else vv) for kk, vv in v.items()} for k, v in stages.items()},
+    }
+    if not args.no_cpu:
+        if w.fp8:
+            record["cpu_baseline"] = {"value": None, "unit": "tokens/s", "cores": 0, "kind": "port",
+                                      "sample": "not run: the CPU path has no fp8 form"}
+        else:
+            record["cpu_baseline"] = _cpu_baseline(w, x, ids, gates, layer)
+    print(json.dumps(record), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -6,7 +6,8 @@ import os
 from ctypes import c_char_p, c_int, c_int64, c_size_t, c_void_p, POINTER
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libdmoe_hip.so")
+# DMOE_HIP_LIB selects an experimental build of the same library (tuning only)
+LIB_PATH = os.environ.get("DMOE_HIP_LIB") or os.path.join(_HERE, "libdmoe_hip.so")
 
 # dmoe.h constants
 OK = 0

@@ -14,7 +14,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_PATH = os.path.join(HERE, "libdmoe_hip.so")
-SOURCES = ["route.hip", "rows.hip", "gmm.hip"]
+SOURCES = ["route.hip", "rows.hip", "gmm.hip", "gmm_direct.hip"]
 ARCH = "gfx950"
 
 FLAGS = [
@@ -31,9 +31,11 @@ def _hipcc() -> str:
     return exe
 
 
-def build(verbose: bool = True, jobs: int = 4, extra_flags=()) -> str:
+def build(verbose: bool = True, jobs: int = 4, extra_flags=(), out: str = LIB_PATH, tag: str = "") -> str:
+    """Compile and link; ``extra_flags``/``out``/``tag`` build an experimental copy
+    next to the default library (select it with the DMOE_HIP_LIB environment variable)."""
     hipcc = _hipcc()
-    objdir = os.path.join(HERE, "build")
+    objdir = os.path.join(HERE, "build" + tag)
     os.makedirs(objdir, exist_ok=True)
 
     def compile_one(src: str) -> str:
@@ -53,16 +55,22 @@ def build(verbose: bool = True, jobs: int = 4, extra_flags=()) -> str:
 
     with ThreadPoolExecutor(max_workers=jobs) as pool:
         objs = list(pool.map(compile_one, SOURCES))
-    tmp = LIB_PATH + ".tmp"
+    tmp = out + ".tmp"
     cmd = [hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-fno-gpu-rdc", *objs, "-o", tmp]
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError(f"link failed:\n{res.stdout}\n{res.stderr}")
-    os.replace(tmp, LIB_PATH)
-    return LIB_PATH
+    os.replace(tmp, out)
+    return out
 
 
 if __name__ == "__main__":
-    print(build())
+    import argparse
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--tag", default="", help="suffix of an experimental library (libdmoe_hip<tag>.so)")
+    ap.add_argument("flags", nargs="*", help="extra hipcc flags, e.g. -DDMOE_SWZ_MODE=1")
+    a, unknown = ap.parse_known_args()
+    target = LIB_PATH if not a.tag else LIB_PATH.replace(".so", a.tag + ".so")
+    print(build(extra_flags=tuple(a.flags) + tuple(unknown), out=target, tag=a.tag))

@@ -17,37 +17,14 @@
 //     its way into LDS so that both MFMA operands are read K-contiguous;
 //   * each wavefront owns a TM x TN sub-tile as FM x FN accumulators of
 //     v_mfma_f32_32x32x16_bf16 (v_mfma_f32_32x32x64_f8f6f4 for fp8).
-#include <type_traits>
-
-#include "common.h"
+#include "gmm_common.h"
 
 namespace dmoe {
 
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-typedef int i32x8 __attribute__((ext_vector_type(8)));
-
-constexpr int kMaxGroups = 1024;   // experts per call (LDS tables)
 constexpr int kRowBytes = 128;     // bytes of K per tile row in LDS
-constexpr int kXcds = 8;
-
-struct GmmArgs {
-    const char *a;
-    const char *b;
-    char *c;
-    const int64_t *batch_sizes;
-    const float *a_scale;
-    const float *b_scale;
-    int64_t rows;   // rows of a / c
-    int E;
-    int K;          // contraction length (elements)
-    int N;          // columns of b per expert (2*I for the swiglu form)
-    int ldc;        // columns of c (N, or I for the swiglu form)
-};
 
 #ifndef DMOE_SWZ_MODE
-#define DMOE_SWZ_MODE 0
+#define DMOE_SWZ_MODE 1
 #endif
 // XOR applied to the 16-byte chunk index of a 128-byte LDS row.  Both forms have
 // a period of at most 32 rows, so fragment rows 32 apart differ by a constant.
@@ -70,7 +47,8 @@ void gmm_kernel(const GmmArgs p) {
     constexpr int KR = BK * (BN / 8) / NT;       // [E,K,N] layout: k-rows of one 8-column group per thread
     constexpr int KG = BK / KR;                  // such groups along K
     constexpr bool FRAG_DB = (WM * WN == 4);     // one wave per SIMD: double-buffer the MFMA operands
-    constexpr int SLOTS = FRAG_DB ? 2 : 1;
+    constexpr int STEP_KS = FP8 ? 1 : 2;         // two waves per SIMD: MFMA k-steps per ping-pong phase
+    constexpr int SLOTS = FRAG_DB ? 2 : STEP_KS;
     static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "wave tile");
     static_assert(CA >= 1 && CB >= 1 && (BM * 8) % NT == 0 && (BN * 8) % NT == 0, "staging split");
     static_assert(RSTEP % 32 == 0 && (BN / 2) % RSTEP == 0, "staging rows keep their swizzle and their half");
@@ -91,43 +69,7 @@ void gmm_kernel(const GmmArgs p) {
     const int wm = wave / WN, wn = wave % WN;
     const int E = p.E;
 
-    // ---- work list: prefix sums of rows and m-tiles over the experts ----
-    if (wave == 0) {
-        long long row_carry = 0;
-        int tile_carry = 0;
-        for (int e0 = 0; e0 < E; e0 += kWave) {
-            const int e = e0 + lane;
-            long long n = (e < E) ? (long long)p.batch_sizes[e] : 0;
-            n = n < 0 ? 0 : (n > p.rows ? p.rows : n);
-            long long incl = n;
-#pragma unroll
-            for (int s = 1; s < kWave; s <<= 1) {
-                long long up = __shfl_up(incl, s, kWave);
-                if (lane >= s) incl += up;
-            }
-            long long start = row_carry + incl - n;
-            if (start > p.rows) start = p.rows;
-            long long end = row_carry + incl;
-            if (end > p.rows) end = p.rows;
-            const int mt = (int)((end - start + BM - 1) / BM);
-            int tincl = mt;
-#pragma unroll
-            for (int s = 1; s < kWave; s <<= 1) {
-                int up = __shfl_up(tincl, s, kWave);
-                if (lane >= s) tincl += up;
-            }
-            if (e < E) {
-                s_row_start[e] = (int)start;
-                s_tile_start[e] = tile_carry + tincl - mt;
-            }
-            row_carry += __shfl(incl, kWave - 1, kWave);
-            tile_carry += __shfl(tincl, kWave - 1, kWave);
-        }
-        if (lane == 0) {
-            s_row_start[E] = (int)(row_carry > p.rows ? p.rows : row_carry);
-            s_tile_start[E] = tile_carry;
-        }
-    }
+    build_work_list<BM>(p, s_tile_start, s_row_start);
     __syncthreads();
 
     const int n_out = SWIGLU ? p.N / 2 : p.N;            // output columns
@@ -136,7 +78,6 @@ void gmm_kernel(const GmmArgs p) {
     const long long total = (long long)m_tiles * n_tiles;
     const int KT = (p.K * ES + kRowBytes - 1) / kRowBytes;
     const int G = gridDim.x;
-    const long long full_rounds = (G % kXcds == 0) ? total / G : 0;  // rounds in which the XCD remap is a bijection
     const uint32_t a_pitch = (uint32_t)(p.K * ES);       // bytes per row of a (and of b when K-contiguous)
 
     // per-thread staging coordinates
@@ -154,39 +95,26 @@ void gmm_kernel(const GmmArgs p) {
     const int fsw = swz(l31);
 
     for (long long q = blockIdx.x; q < total; q += G) {
-        // ---- decode the work item ----
-        long long L = q;
-        const long long round = q / G;
-        if (round < full_rounds) {
-            const int w = (int)(q - round * G);
-            L = round * G + (long long)(w % kXcds) * (G / kXcds) + (w / kXcds);
-        }
-        const int u = (int)(L / n_tiles);
-        int lo = 0, hi = E;  // last e with s_tile_start[e] <= u
-        while (hi - lo > 1) {
-            const int mid = (lo + hi) >> 1;
-            if (s_tile_start[mid] <= u) lo = mid; else hi = mid;
-        }
-        const int e = lo;
-        const int mt_e = s_tile_start[e + 1] - s_tile_start[e];
-        const int local = (int)(L - (long long)s_tile_start[e] * n_tiles);
-        const int nt = local / mt_e;
-        const int mi = local - nt * mt_e;
-        const int row0 = s_row_start[e] + mi * BM;             // first row of the tile
-        const int rows_e = s_row_start[e + 1] - row0;          // valid rows from row0 on (>= 1)
+        const TileCoord tc = decode_tile<BM>(q, G, total, n_tiles, E, s_tile_start, s_row_start);
+        const int e = tc.e, nt = tc.nt, row0 = tc.row0, rows_e = tc.rows_e;
         const int n0 = nt * BNO;                               // first output column
 
         // ---- staging offsets (bytes from wave-uniform bases) ----
         const char *a_base = p.a + (long long)row0 * a_pitch;
         const char *b_exp = p.b + (long long)e * p.K * p.N * ES;
-        // first column of the tile's two halves (plain form: one "half" of BN columns)
+#ifdef DMOE_DBG_SAME_B
+        const int n0_b = 0;       // timing experiment: every n-tile reads the first weight tile (wrong results)
+#else
+        const int n0_b = n0;
+#endif
+        // first column of the tile; the swiglu form reads a second run of columns (the up half)
         const char *b_base0, *b_base1;
         if constexpr (TRANS_B) {
-            b_base0 = b_exp + (long long)n0 * a_pitch;
-            b_base1 = SWIGLU ? b_exp + (long long)(n_out + n0) * a_pitch : b_base0 + (long long)(BN / 2) * a_pitch;
+            b_base0 = b_exp + (long long)n0_b * a_pitch;
+            b_base1 = SWIGLU ? b_exp + (long long)(n_out + n0_b) * a_pitch : b_base0;
         } else {
-            b_base0 = b_exp + (long long)n0 * ES;
-            b_base1 = SWIGLU ? b_exp + (long long)(n_out + n0) * ES : b_base0 + (BN / 2) * ES;
+            b_base0 = b_exp + (long long)n0_b * ES;
+            b_base1 = SWIGLU ? b_exp + (long long)(n_out + n0_b) * ES : b_base0;
         }
         const int half_cols = SWIGLU ? n_out - n0 : p.N - n0;  // valid columns from the first column of half 0
         uint32_t a_off[CA];
@@ -202,17 +130,15 @@ void gmm_kernel(const GmmArgs p) {
 #pragma unroll
             for (int i = 0; i < CB; ++i) {
                 const int r = a_row0 + i * RSTEP;              // row of the B tile = output column slot
-                const int rh = (r < BN / 2) ? r : r - BN / 2;  // column inside its half
-                const bool ok = SWIGLU ? rh < half_cols : r < half_cols;
-                b_off[i] = (uint32_t)(ok ? rh : 0) * a_pitch + a_chunk * 16;
+                const int rh = (SWIGLU && r >= BN / 2) ? r - BN / 2 : r;  // column from its base
+                b_off[i] = (uint32_t)(rh < half_cols ? rh : 0) * a_pitch + a_chunk * 16;
             }
         } else {
             const int r = b_ng * 8;                            // first of 8 columns, all in one half
-            const int rh = (r < BN / 2) ? r : r - BN / 2;
-            const bool ok = SWIGLU ? rh < half_cols : r < half_cols;  // N % 8 == 0: valid together
-            b_off[0] = (uint32_t)(ok ? rh : 0) * ES;
+            const int rh = (SWIGLU && r >= BN / 2) ? r - BN / 2 : r;
+            b_off[0] = (uint32_t)(rh < half_cols ? rh : 0) * ES;   // N % 8 == 0: the 8 columns are valid together
         }
-        const bool b_hi_half = !TRANS_B && (b_ng * 8 >= BN / 2);
+        const bool b_hi_half = !TRANS_B && SWIGLU && (b_ng * 8 >= BN / 2);
 
         u32x4 ra[CA], rb[CB];
         // kTail: the tile reaches past K; bytes past the end of a row are read as zero
@@ -228,7 +154,7 @@ void gmm_kernel(const GmmArgs p) {
             if constexpr (TRANS_B) {
 #pragma unroll
                 for (int i = 0; i < CB; ++i) {
-                    const char *bk = ((i * RSTEP < BN / 2) ? b_base0 : b_base1) + (long long)kt * kRowBytes;
+                    const char *bk = ((SWIGLU && i * RSTEP >= BN / 2) ? b_base1 : b_base0) + (long long)kt * kRowBytes;
                     if (kTail) rb[i] = u32x4{0, 0, 0, 0};
                     if (k_ok) rb[i] = *(const u32x4 *)(bk + b_off[i]);
                 }
@@ -244,6 +170,9 @@ void gmm_kernel(const GmmArgs p) {
         };
         const int KT_full = (p.K * ES) / kRowBytes;            // tiles that lie inside K entirely
         auto load_tile = [&](int kt) {
+#ifdef DMOE_DBG_NO_GLOAD
+            if (kt > 1) return;   // timing experiment: no global traffic after the prologue (wrong results)
+#endif
             if (kt < KT_full) load_global(kt, std::false_type{});
             else load_global(kt, std::true_type{});
         };
@@ -353,11 +282,11 @@ void gmm_kernel(const GmmArgs p) {
         if constexpr (FRAG_DB) load_frags(0, 0, 0);
 
         // ---- main loop over K tiles ----
-        for (int kt = 0; kt < KT; ++kt) {
-            const int cur = kt & 1;
+        if constexpr (FRAG_DB) {
+            for (int kt = 0; kt < KT; ++kt) {
+                const int cur = kt & 1;
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
-                if constexpr (FRAG_DB) {
+                for (int ks = 0; ks < KS; ++ks) {
                     const int slot = ks & 1;
                     if (ks + 1 < KS) load_frags(cur, ks + 1, slot ^ 1);
                     if (ks == KS - 2) {
@@ -369,17 +298,40 @@ void gmm_kernel(const GmmArgs p) {
                         if (kt + 1 < KT) load_frags(cur ^ 1, 0, slot ^ 1);
                     }
                     mfma_all(acc, slot);
-                } else {
-                    // two waves per SIMD cover each other's LDS latency: operands are read just in time
-                    load_frags(cur, ks, 0);
-                    if (ks == KS - 2) {
+                }
+            }
+        } else {
+            // Two waves share a SIMD.  The two halves of the workgroup run half a step apart: while one
+            // half issues its LDS/global traffic for a step, the other half issues the MFMAs of its step,
+            // and the barriers hand the roles over.  Waves w and w + 4 sit on the same SIMD.
+#ifndef DMOE_PP_GROUP_MODE
+#define DMOE_PP_GROUP_MODE 0
+#endif
+            const int grp = DMOE_PP_GROUP_MODE == 0 ? (wave >> 2) : (wave & 1);
+            if (grp == 1) __syncthreads();
+            for (int kt = 0; kt < KT; ++kt) {
+                const int cur = kt & 1;
+#pragma unroll
+                for (int st = 0; st < KS / STEP_KS; ++st) {
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int u = 0; u < STEP_KS; ++u) load_frags(cur, st * STEP_KS + u, u);
+                    if (st == 0) {
                         if (kt + 1 < KT) store_lds(cur ^ 1);
                         if (kt + 2 < KT) load_tile(kt + 2);
                     }
-                    mfma_all(acc, 0);
-                    if (ks == KS - 1) __syncthreads();
+                    __builtin_amdgcn_sched_barrier(0);
+                    __syncthreads();
+                    __builtin_amdgcn_sched_barrier(0);
+                    __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+                    for (int u = 0; u < STEP_KS; ++u) mfma_all(acc, u);
+                    __builtin_amdgcn_s_setprio(0);
+                    __builtin_amdgcn_sched_barrier(0);
+                    __syncthreads();
                 }
             }
+            if (grp == 0) __syncthreads();
         }
 
         // ---- epilogue: accumulator (row, col) = ((x/4)*8 + (lane/32)*4 + x%4, lane%32) ----
@@ -439,17 +391,26 @@ static int launch_one(const GmmArgs &args, hipStream_t stream) {
     return DMOE_OK;
 }
 
-static int g_variant = 0;  // 0: 8 wavefronts per 256x256 tile, 1: 4 wavefronts
+static int g_variant = 0;  // tuning hook, see dmoe_gmm_tune
 
 template <bool TRANS_B, bool SWIGLU, bool FP8>
 static int launch_by_rows(const GmmArgs &args, hipStream_t stream) {
     // rows per expert on average decide the m-tile; the host does not know the split
     const long long avg = args.rows / (args.E > 0 ? args.E : 1);
-    if (g_variant == 2) return launch_one<64, 256, 1, 4, TRANS_B, SWIGLU, FP8>(args, stream);
-    if (g_variant == 3) return launch_one<128, 256, 1, 4, TRANS_B, SWIGLU, FP8>(args, stream);
-    if (avg <= 64 && g_variant == 0) return launch_one<64, 256, 1, 4, TRANS_B, SWIGLU, FP8>(args, stream);
-    if (avg <= 160 && g_variant == 0) return launch_one<128, 256, 1, 4, TRANS_B, SWIGLU, FP8>(args, stream);
-    if (g_variant == 1) return launch_one<256, 256, 2, 2, TRANS_B, SWIGLU, FP8>(args, stream);
+    switch (g_variant) {
+        case 1: return launch_one<256, 256, 2, 2, TRANS_B, SWIGLU, FP8>(args, stream);
+        case 2: return launch_one<64, 256, 1, 4, TRANS_B, SWIGLU, FP8>(args, stream);
+        case 3: return launch_one<128, 256, 1, 4, TRANS_B, SWIGLU, FP8>(args, stream);
+        case 4: return launch_one<256, 256, 2, 4, TRANS_B, SWIGLU, FP8>(args, stream);
+        default: break;
+    }
+    if (avg <= 64) return launch_one<64, 256, 1, 4, TRANS_B, SWIGLU, FP8>(args, stream);
+    if (avg <= 160) return launch_one<128, 256, 1, 4, TRANS_B, SWIGLU, FP8>(args, stream);
+    if constexpr (!FP8) {
+        // global -> LDS direct path: whole stages of 32 k, 32-bit offsets inside one expert's weights
+        if (args.K % 32 == 0 && (long long)args.K * args.N * 2 < (1ll << 32))
+            return launch_direct_bf16(args, TRANS_B, SWIGLU, stream);
+    }
     return launch_one<256, 256, 2, 4, TRANS_B, SWIGLU, FP8>(args, stream);
 }
 
@@ -471,7 +432,7 @@ static int check_gmm(const char *who, const void *a, const void *b, const void *
 using namespace dmoe;
 
 extern "C" int dmoe_gmm_tune(int variant) {
-    DMOE_REQUIRE(variant >= 0 && variant <= 3, DMOE_ERR_ARG, "dmoe_gmm_tune: variant %d outside [0, 3]", variant);
+    DMOE_REQUIRE(variant >= 0 && variant <= 4, DMOE_ERR_ARG, "dmoe_gmm_tune: variant %d outside [0, 4]", variant);
     g_variant = variant;
     return DMOE_OK;
 }

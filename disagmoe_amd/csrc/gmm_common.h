@@ -1,0 +1,116 @@
+// Pieces shared by the grouped GEMM kernels: argument block, vector types and the
+// device-side work list (expert, m-tile, n-tile) derived from batch_sizes.
+#pragma once
+
+#include <type_traits>
+
+#include "common.h"
+
+namespace dmoe {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+
+constexpr int kMaxGroups = 1024;   // experts per call (LDS tables)
+constexpr int kXcds = 8;
+
+struct GmmArgs {
+    const char *a;
+    const char *b;
+    char *c;
+    const int64_t *batch_sizes;
+    const float *a_scale;
+    const float *b_scale;
+    int64_t rows;   // rows of a / c
+    int E;
+    int K;          // contraction length (elements)
+    int N;          // columns of b per expert (2*I for the swiglu form)
+    int ldc;        // columns of c (N, or I for the swiglu form)
+};
+
+// Prefix sums of rows and m-tiles over the experts, built by the first wavefront
+// into LDS tables of E + 1 entries.  Sizes are clamped so that the running row
+// count never passes p.rows.  The caller synchronises the workgroup afterwards.
+template <int BM>
+__device__ __forceinline__ void build_work_list(const GmmArgs &p, int *s_tile_start, int *s_row_start) {
+    const int lane = threadIdx.x & (kWave - 1);
+    if (threadIdx.x >= kWave) return;
+    const int E = p.E;
+    long long row_carry = 0;
+    int tile_carry = 0;
+    for (int e0 = 0; e0 < E; e0 += kWave) {
+        const int e = e0 + lane;
+        long long n = (e < E) ? (long long)p.batch_sizes[e] : 0;
+        n = n < 0 ? 0 : (n > p.rows ? p.rows : n);
+        long long incl = n;
+#pragma unroll
+        for (int s = 1; s < kWave; s <<= 1) {
+            long long up = __shfl_up(incl, s, kWave);
+            if (lane >= s) incl += up;
+        }
+        long long start = row_carry + incl - n;
+        if (start > p.rows) start = p.rows;
+        long long end = row_carry + incl;
+        if (end > p.rows) end = p.rows;
+        const int mt = (int)((end - start + BM - 1) / BM);
+        int tincl = mt;
+#pragma unroll
+        for (int s = 1; s < kWave; s <<= 1) {
+            int up = __shfl_up(tincl, s, kWave);
+            if (lane >= s) tincl += up;
+        }
+        if (e < E) {
+            s_row_start[e] = (int)start;
+            s_tile_start[e] = tile_carry + tincl - mt;
+        }
+        row_carry += __shfl(incl, kWave - 1, kWave);
+        tile_carry += __shfl(tincl, kWave - 1, kWave);
+    }
+    if (lane == 0) {
+        s_row_start[E] = (int)(row_carry > p.rows ? p.rows : row_carry);
+        s_tile_start[E] = tile_carry;
+    }
+}
+
+struct TileCoord {
+    int e;        // expert
+    int nt;       // n-tile
+    int row0;     // first row of the tile in a / c
+    int rows_e;   // rows of the expert from row0 on (>= 1; the tile holds min(rows_e, BM) of them)
+};
+
+// Work item q of workgroup-strided order -> tile.  Consecutive blocks of G/8 items go to the
+// workgroups of one XCD (workgroup id % 8); inside an expert the order is m-fastest, so the
+// m-tiles that share a weight tile run next to each other on one L2.
+template <int BM>
+__device__ __forceinline__ TileCoord decode_tile(long long q, int G, long long total, int n_tiles, int E,
+                                                 const int *s_tile_start, const int *s_row_start) {
+    long long L = q;
+    const long long full_rounds = (G % kXcds == 0) ? total / G : 0;  // rounds in which the remap is a bijection
+    const long long round = q / G;
+    if (round < full_rounds) {
+        const int w = (int)(q - round * G);
+        L = round * G + (long long)(w % kXcds) * (G / kXcds) + (w / kXcds);
+    }
+    const int u = (int)(L / n_tiles);
+    int lo = 0, hi = E;  // last e with s_tile_start[e] <= u
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (s_tile_start[mid] <= u) lo = mid; else hi = mid;
+    }
+    TileCoord t;
+    t.e = lo;
+    const int mt_e = s_tile_start[lo + 1] - s_tile_start[lo];
+    const int local = (int)(L - (long long)s_tile_start[lo] * n_tiles);
+    t.nt = local / mt_e;
+    const int mi = local - t.nt * mt_e;
+    t.row0 = s_row_start[lo] + mi * BM;
+    t.rows_e = s_row_start[lo + 1] - t.row0;
+    return t;
+}
+
+int launch_direct_bf16(const GmmArgs &args, bool trans_b, bool swiglu, hipStream_t stream);
+
+}  // namespace dmoe

@@ -1,0 +1,275 @@
+// bf16 grouped GEMM, 256x256 tiles, for row counts that fill them: the CDNA4 data path.
+//
+//   * A and B tiles go global -> LDS directly (global_load_lds_dwordx4: each lane
+//     fetches 16 bytes, the wavefront fills 1 KiB of LDS), no staging registers,
+//     no LDS store instructions;
+//   * K is cut in stages of 32; four stages of 32 KiB live in LDS, so a load is
+//     issued three stages (about 3000 MFMA cycles) before its data is needed;
+//   * the LDS images are permuted on the way in (the lane picks WHICH 16 bytes of
+//     the row it fetches) so that the operand reads are bank-conflict free:
+//       - K-contiguous operands ([rows][32 k] = 64 B rows): chunk ^ ((row >> 2) & 3),
+//         read with ds_read_b128;
+//       - B in the [K, N] layout is kept [k][256 n] (512 B rows): chunk ^ ((k & 3) << 2),
+//         read with ds_read_b64_tr_b16, which transposes 4 k x 16 n inside 16 lanes
+//         and hands every lane 4 consecutive k of its column - the MFMA B operand;
+//   * 4 wavefronts, one per SIMD, each owns 128x128 of the tile as 4x4
+//     v_mfma_f32_32x32x16_bf16 accumulators; operands are double buffered in
+//     registers one k-step ahead; one workgroup barrier per stage.
+#include "gmm_common.h"
+
+namespace dmoe {
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+#define DMOE_LDS_PTR(p) ((__attribute__((address_space(3))) void *)(p))
+
+// One wavefront copies 64 x 16 bytes from per-lane global addresses to 1 KiB of LDS at `lds`
+// (wave-uniform byte address, goes through M0).  Written as asm so that the compiler does not
+// serialise later LDS reads behind every outstanding copy; completion is tracked by hand
+// with vmcnt (the copies complete in issue order).
+__device__ __forceinline__ void copy_g2lds_16(const char *gptr, uint32_t lds) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                 :: "v"(gptr), "s"(__builtin_amdgcn_readfirstlane(lds)) : "memory", "m0");
+}
+__device__ __forceinline__ uint32_t lds_addr(const void *p) { return (uint32_t)(uintptr_t)DMOE_LDS_PTR(p); }
+
+constexpr int kDM = 256, kDN = 256;        // tile
+constexpr int kDK = 32;                    // k per stage
+constexpr int kStages = 4;
+constexpr int kStageA = kDM * kDK * 2;     // 16 KiB
+constexpr int kStageB = kDN * kDK * 2;     // 16 KiB
+constexpr int kStage = kStageA + kStageB;
+constexpr int kLoads = 8;                  // global_load_lds per wavefront per stage (4 A + 4 B)
+
+// s_waitcnt with only vmcnt set (gfx9 encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14)
+#define DMOE_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (7 << 4) | (15 << 8) | (((n) >> 4) << 14))
+
+template <bool TRANS_B, bool SWIGLU>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void gmm_direct_kernel(const GmmArgs p) {
+    constexpr int BNO = SWIGLU ? kDN / 2 : kDN;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    __shared__ int s_tile_start[kMaxGroups + 1];
+    __shared__ int s_row_start[kMaxGroups + 1];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int E = p.E;
+
+    build_work_list<kDM>(p, s_tile_start, s_row_start);
+    __syncthreads();
+
+    const int n_out = SWIGLU ? p.N / 2 : p.N;
+    const int n_tiles = (n_out + BNO - 1) / BNO;
+    const long long total = (long long)s_tile_start[E] * n_tiles;
+    const int S = p.K / kDK;                       // stages (K % 32 == 0)
+    const int G = gridDim.x;
+    const uint32_t pitch = (uint32_t)p.K * 2;      // bytes per row of a (and of b when K-contiguous)
+    const uint32_t smem_addr = lds_addr(smem);
+
+    // ---- per-lane constants of the global -> LDS copies ----
+    // K-contiguous image: a 1 KiB block is 16 rows of 64 B; lane l fills row l/4, physical chunk l%4
+    const int kc_row = lane >> 2;
+    const int kc_chunk = (lane & 3) ^ ((lane >> 4) & 3);      // logical chunk stored there
+    // [k][n] image: a 1 KiB block is 2 k-rows of 512 B; lane l fills k-row l/32, physical chunk l%32
+    const int kn_k = 2 * wave + (lane >> 5);                  // k inside the stage, block i adds 8 i
+    const int kn_chunk = (lane & 31) ^ ((kn_k & 3) << 2);     // logical chunk (8 columns) stored there
+
+    // ---- per-lane constants of the operand reads ----
+    const int l31 = lane & 31, kgrp = lane >> 5;
+    const int fa_base = (wm * 128 + l31) * 64;
+    const int f_sw = (l31 >> 2) & 3;
+    const int g16 = lane >> 4, i16 = lane & 15;
+
+    for (long long q = blockIdx.x; q < total; q += G) {
+        const TileCoord tc = decode_tile<kDM>(q, G, total, n_tiles, E, s_tile_start, s_row_start);
+        const int e = tc.e, row0 = tc.row0, rows_e = tc.rows_e;
+        const int n0 = tc.nt * BNO;
+        const int half_cols = n_out - n0;                      // valid columns from n0 on
+
+        // tile column slot (0..255) -> column of b; slots past the end read column n0 (never stored)
+        auto b_col = [&](int slot) {
+            const int rh = (SWIGLU && slot >= kDN / 2) ? slot - kDN / 2 : slot;
+            const int base = (SWIGLU && slot >= kDN / 2) ? n_out + n0 : n0;
+            return base + (rh < half_cols ? rh : 0);
+        };
+
+        const char *a_base = p.a + (long long)row0 * pitch;
+        const char *b_exp = p.b + (long long)e * p.K * p.N * 2;
+        uint32_t a_off[4], b_off[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            int r = (i * 4 + wave) * 16 + kc_row;
+            if (r >= rows_e) r = rows_e - 1;                   // clamp: loaded, never stored
+            a_off[i] = (uint32_t)r * pitch + kc_chunk * 16;
+            if constexpr (TRANS_B) b_off[i] = (uint32_t)b_col((i * 4 + wave) * 16 + kc_row) * pitch + kc_chunk * 16;
+        }
+        if constexpr (!TRANS_B) b_off[0] = (uint32_t)kn_k * (uint32_t)p.N * 2 + (uint32_t)b_col(kn_chunk * 8) * 2;
+
+        auto issue_loads = [&](int s) {
+            const uint32_t lA = smem_addr + (s & (kStages - 1)) * kStage + wave * 1024;
+            const uint32_t lB = lA + kStageA;
+            const char *ga = a_base + (long long)s * (kDK * 2);
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                copy_g2lds_16(ga + a_off[i], lA + i * 4096);
+            if constexpr (TRANS_B) {
+                const char *gb = b_exp + (long long)s * (kDK * 2);
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    copy_g2lds_16(gb + b_off[i], lB + i * 4096);
+            } else {
+                const char *gb = b_exp + (long long)s * kDK * p.N * 2 + b_off[0];
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    copy_g2lds_16(gb + (long long)i * 8 * p.N * 2, lB + i * 4096);
+            }
+        };
+
+        // B operand rows / columns of this wavefront: fragment j covers 32 tile columns
+        int fb_off[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int slot0 = SWIGLU ? ((j < 2) ? wn * 64 + j * 32 : kDN / 2 + wn * 64 + (j - 2) * 32) : wn * 128 + j * 32;
+            if constexpr (TRANS_B) {
+                fb_off[j] = (slot0 + l31) * 64;
+            } else {
+                const int col = slot0 + (g16 & 1) * 16 + 4 * (i16 & 3);          // tile column of this lane's 4 values
+                const int chunk = (col >> 3) ^ (((i16 >> 2) & 3) << 2);
+                fb_off[j] = ((kgrp * 8) + (i16 >> 2)) * 512 + chunk * 16 + (col & 7) * 2;
+            }
+        }
+
+        bf16x8 fa[2][4], fb[2][4];
+        auto load_frags = [&](int s, int ks, int slot) {
+            const char *tA = smem + (s & (kStages - 1)) * kStage;
+            const char *tB = tA + kStageA;
+            const int c0 = ((ks * 2 + kgrp) ^ f_sw) << 4;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const u32x4 x = *(const u32x4 *)(tA + fa_base + i * 2048 + c0);
+                __builtin_memcpy(&fa[slot][i], &x, 16);
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if constexpr (TRANS_B) {
+                    const u32x4 x = *(const u32x4 *)(tB + fb_off[j] + c0);
+                    __builtin_memcpy(&fb[slot][j], &x, 16);
+                } else {
+                    const char *src = tB + fb_off[j] + ks * (16 * 512);
+                    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)DMOE_LDS_PTR(src));
+                    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)DMOE_LDS_PTR(src + 4 * 512));
+                    const s16x8 v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                    __builtin_memcpy(&fb[slot][j], &v, 16);
+                }
+            }
+        };
+
+        f32x16 acc[4][4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int x = 0; x < 16; ++x) acc[i][j][x] = 0.f;
+        auto mfma_all = [&](int slot) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[slot][i], fb[slot][j], acc[i][j], 0, 0, 0);
+        };
+
+        // ---- prologue: every LDS stage is free (the previous tile ended with a barrier after its last read) ----
+        const int pre = S < kStages ? S : kStages;
+        for (int s = 0; s < pre; ++s) issue_loads(s);
+        if (pre == 4) DMOE_WAIT_VMCNT(3 * kLoads);
+        else if (pre == 3) DMOE_WAIT_VMCNT(2 * kLoads);
+        else if (pre == 2) DMOE_WAIT_VMCNT(kLoads);
+        else DMOE_WAIT_VMCNT(0);
+        __syncthreads();
+        load_frags(0, 0, 0);
+
+        // One stage: k-step 0, then k-step 1 with the hand-over to stage s+1 behind its first MFMAs.
+        // kAhead = stages after s+1 whose copies are already in flight (they may still be when s+1 is opened).
+        auto run_stage = [&](int s, auto ahead_tag, auto next_tag) {
+            constexpr int kAhead = decltype(ahead_tag)::value;
+            constexpr bool kNext = decltype(next_tag)::value;
+            load_frags(s, 1, 1);
+            __builtin_amdgcn_sched_barrier(0);      // keep the operand reads ahead of the MFMAs that hide them
+            mfma_all(0);
+            __builtin_amdgcn_sched_barrier(0);      // the hand-over below stays behind these MFMAs
+            if constexpr (kNext) {
+                DMOE_WAIT_VMCNT(kAhead * kLoads);   // this wavefront's share of stage s+1 has landed ...
+                __syncthreads();                    // ... so has everybody else's; all reads of stage s are done
+                if (s + kStages < S) issue_loads(s + kStages);   // refill the stage just drained
+                load_frags(s + 1, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            mfma_all(1);
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        int s = 0;
+        for (; s + 3 < S; ++s) run_stage(s, std::integral_constant<int, 2>{}, std::true_type{});
+        if (s + 2 < S) { run_stage(s, std::integral_constant<int, 1>{}, std::true_type{}); ++s; }
+        if (s + 1 < S) { run_stage(s, std::integral_constant<int, 0>{}, std::true_type{}); ++s; }
+        run_stage(s, std::integral_constant<int, 0>{}, std::false_type{});
+        __syncthreads();   // the last stage has been read by everyone before the next tile refills LDS
+
+        // ---- epilogue: accumulator (row, col) = ((x/4)*8 + (lane/32)*4 + x%4, lane%32) ----
+        uint16_t *cbase = (uint16_t *)p.c;
+        constexpr int FNO = SWIGLU ? 2 : 4;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+#pragma unroll
+            for (int j = 0; j < FNO; ++j) {
+                const int ccol = n0 + (SWIGLU ? wn * 64 : wn * 128) + j * 32 + l31;
+                if (ccol >= n_out) continue;
+#pragma unroll
+                for (int x = 0; x < 16; ++x) {
+                    const int r = wm * 128 + i * 32 + (x >> 2) * 8 + kgrp * 4 + (x & 3);
+                    if (r >= rows_e) continue;
+                    float v;
+                    if (SWIGLU) {
+                        const float g = acc[i][j][x];
+                        v = g / (1.f + __expf(-g)) * acc[i][j + 2][x];
+                    } else {
+                        v = acc[i][j][x];
+                    }
+                    cbase[(long long)(row0 + r) * p.ldc + ccol] = f32_to_bf16(v);
+                }
+            }
+        }
+    }
+}
+
+template <bool TRANS_B, bool SWIGLU>
+static int launch_direct_one(const GmmArgs &args, hipStream_t stream) {
+    constexpr int BNO = SWIGLU ? kDN / 2 : kDN;
+    const size_t lds = (size_t)kStages * kStage;
+    auto kern = gmm_direct_kernel<TRANS_B, SWIGLU>;
+    static bool configured = false;
+    if (!configured) {
+        DMOE_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        configured = true;
+    }
+    const int n_out = SWIGLU ? args.N / 2 : args.N;
+    const long long n_tiles = (n_out + BNO - 1) / BNO;
+    const long long m_tiles_max = args.rows / kDM + args.E;
+    long long grid = (long long)device_cus();
+    if (m_tiles_max * n_tiles < grid) grid = m_tiles_max * n_tiles;
+    if (grid < 1) grid = 1;
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), lds, stream, args);
+    DMOE_LAUNCH_CHECK("gmm_direct_kernel");
+    return DMOE_OK;
+}
+
+// Preconditions (checked by the caller): bf16, K % 32 == 0, N % 8 == 0, K * N * 2 < 2^32.
+int launch_direct_bf16(const GmmArgs &args, bool trans_b, bool swiglu, hipStream_t stream) {
+    if (trans_b) return swiglu ? launch_direct_one<true, true>(args, stream) : launch_direct_one<true, false>(args, stream);
+    return swiglu ? launch_direct_one<false, true>(args, stream) : launch_direct_one<false, false>(args, stream);
+}
+
+}  // namespace dmoe

@@ -117,17 +117,17 @@ def quantize_rows(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
 
 
 def quantize_weight(w: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
-    """Offline weight quantisation (torch ops, not on the hot path): ``w [E, K,
-    N]`` -> ``(q [E, N, K] float8_e4m3fn, scale [E, N] fp32)``, per output channel
-    ``scale = absmax_k / 448``."""
+    """Offline weight quantisation: ``w [E, K, N]`` -> ``(q [E, N, K]
+    float8_e4m3fn, scale [E, N] fp32)``, per output channel ``scale = absmax_k /
+    448``.  An output channel is a row of ``w[e].T``, so the row quantiser does
+    the arithmetic."""
+    assert w.is_cuda and w.dim() == 3
     E, K, N = w.shape
     q = torch.empty((E, N, K), dtype=torch.float8_e4m3fn, device=w.device)
     s = torch.empty((E, N), dtype=torch.float32, device=w.device)
     for e in range(E):
-        wf = w[e].float()
-        se = wf.abs().amax(dim=0) / 448.0
-        se = torch.where(se > 0, se, torch.ones_like(se))
-        q[e] = (wf / se[None, :]).clamp(-448.0, 448.0).t().contiguous().to(torch.float8_e4m3fn)
+        qe, se = quantize_rows(w[e].t().contiguous())
+        q[e] = qe
         s[e] = se
     return q, s
 

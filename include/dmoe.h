@@ -140,8 +140,9 @@ int dmoe_gmm_swiglu(const void *a, const void *b, void *h, const int64_t *batch_
 int dmoe_gmm_workspace_bytes(int E, size_t *bytes);
 
 /* Tuning hook for benchmarks (no counterpart in the reference): 0 = choose the
- * tile shape from rows per expert (default); 1 = 256x256 tile on 4 wavefronts;
- * 2 = 64x256; 3 = 128x256.  Process-wide, not thread-safe. */
+ * kernel from rows per expert (default); 1 = register-staged 256x256 tile on 4
+ * wavefronts; 2 = 64x256; 3 = 128x256; 4 = register-staged 256x256 tile on 8
+ * wavefronts.  Process-wide, not thread-safe. */
 int dmoe_gmm_tune(int variant);
 
 /* ---- fp8 (e4m3) path: no counterpart in the reference ---------------------

@@ -43,3 +43,20 @@ def dequantize_weight(q_nk: torch.Tensor, s: torch.Tensor, dtype=torch.bfloat16)
 
 def dequantize_rows(q: torch.Tensor, s: torch.Tensor, dtype=torch.bfloat16) -> torch.Tensor:
     return (q.detach().cpu().float() * s.detach().cpu().float()[:, None]).to(dtype)
+
+
+def moe_experts_forward_fp8(x: torch.Tensor, q13: torch.Tensor, s13: torch.Tensor, q2: torch.Tensor,
+                            s2: torch.Tensor, batch_sizes) -> torch.Tensor:
+    """The fp8 expert FFN with its quantisation points stated: rows of ``x`` and of
+    the intermediate ``h`` are quantised per token, both GEMMs contract the
+    de-quantised fp8 values in fp32, ``h`` and the result are rounded to bf16."""
+    from . import ffn
+    xq, xs = quantize_rows(x)
+    w13 = dequantize_weight(q13, s13, torch.float32)
+    inter = w13.shape[2] // 2
+    up = ffn.gmm(dequantize_rows(xq, xs, torch.float32), w13, batch_sizes, out_dtype=torch.float32)
+    h = (torch.nn.functional.silu(up[:, :inter]) * up[:, inter:]).to(torch.bfloat16)
+    hq, hs = quantize_rows(h)
+    out = ffn.gmm(dequantize_rows(hq, hs, torch.float32), dequantize_weight(q2, s2, torch.float32), batch_sizes,
+                  out_dtype=torch.float32)
+    return out.to(torch.bfloat16)

@@ -52,7 +52,7 @@ def test_host_side_argument_errors():
     assert lib.dmoe_gmm(None, None, None, None, 16, 8, 60, 64, 0, 0, None) == -2      # K % 8
     assert lib.dmoe_gmm(None, None, None, None, 16, 8, 64, 64, 0, 1, None) == -3      # fp16 not supported
     assert lib.dmoe_gmm_fp8(None, None, None, None, None, None, 16, 8, 72, 64, None) == -2  # K % 16
-    assert lib.dmoe_gmm_tune(9) == -1
+    assert lib.dmoe_gmm_tune(9) == -1 and lib.dmoe_gmm_tune(4) == 0 and lib.dmoe_gmm_tune(0) == 0
     with pytest.raises(_lib.DmoeError):
         _lib.call("dmoe_gmm_tune", -1)
     # empty problems succeed without touching the device

@@ -1,0 +1,125 @@
+"""fp8-e4m3 path.
+
+* The quantiser is bit-exact against the oracle rule.
+* The stated bar, max|out - ref| / max|ref| <= 3e-2: the fp8 GEMM kernels against
+  the oracle gmm on the de-quantised weights, fed the same (fp8-representable)
+  activations the kernel is fed; the FFN against the oracle FFN with the same
+  quantisation points.
+* Against the bf16 oracle on de-quantised weights with UNQUANTISED bf16
+  activations the difference is the rounding of the activations to e4m3 (3
+  mantissa bits: relative step 2^-4, about 2.6 % rms per element, which a dot
+  product of independent terms passes on undiminished).  No fp8-activation kernel
+  can be closer than that; the tests record the figure and bound it at
+  TOL_FP8_ACT."""
+import pytest
+import torch
+
+from disagmoe_amd import workloads
+from disagmoe_amd.grouped_gemm import backend as gg
+from disagmoe_amd.models.experts import MoEExpertsFP8
+from oracle import ffn, fp8
+from helpers import TOL_FP8, announce, dev, max_rel_err, ragged_sizes
+
+pytestmark = pytest.mark.gpu
+
+TOL_FP8_ACT = 8e-2   # activation-rounding noise against the unquantised-activation oracle (see above)
+
+
+@pytest.mark.parametrize("rows,d", [(1, 16), (17, 64), (300, 1024), (64, 6144), (5, 16384)])
+def test_quantize_rows_bit_exact(rows, d):
+    announce(test="quant_rows", rows=rows, d=d)
+    g = torch.Generator().manual_seed(rows + d)
+    x = (torch.randn(rows, d, generator=g) * torch.logspace(-3, 2, rows).view(-1, 1)).to(torch.bfloat16)
+    x[0] = 0
+    q_ref, s_ref = fp8.quantize_rows(x)
+    q, s = gg.quantize_rows(x.to(dev()))
+    assert torch.equal(s.cpu(), s_ref)
+    assert torch.equal(q.cpu().view(torch.uint8), q_ref.view(torch.uint8))
+
+
+def test_quantize_weight_matches_oracle():
+    announce(test="quant_weight")
+    g = torch.Generator().manual_seed(1)
+    w = (torch.randn(3, 128, 96, generator=g) * 0.02).to(torch.bfloat16)
+    q, s = gg.quantize_weight(w.to(dev()))
+    q_ref, s_ref = fp8.quantize_weight_channels(w)
+    assert torch.equal(s.cpu(), s_ref) and torch.equal(q.cpu().view(torch.uint8), q_ref.view(torch.uint8))
+
+
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("E,R,K,N", [(1, 200, 256, 256), (4, 1000, 512, 520), (8, 700, 144, 264)])
+def test_gmm_fp8(variant, E, R, K, N):
+    announce(test="gmm_fp8", variant=variant, E=E, R=R, K=K, N=N)
+    gg.set_tile_variant(variant)
+    try:
+        g = torch.Generator().manual_seed(E + R)
+        a = torch.randn(R, K, generator=g).to(torch.bfloat16)
+        w = (torch.randn(E, K, N, generator=g) * 0.02).to(torch.bfloat16)
+        sizes = ragged_sizes(E, R, seed=R)
+        aq, a_s = fp8.quantize_rows(a)
+        wq, w_s = fp8.quantize_weight_channels(w)
+        out = gg.gmm_fp8(aq.to(dev()), a_s.to(dev()), wq.to(dev()), w_s.to(dev()), sizes)
+        # same quantised operands on both sides: only accumulation order and the output rounding differ
+        exact = ffn.gmm(fp8.dequantize_rows(aq, a_s, torch.float32), fp8.dequantize_weight(wq, w_s, torch.float32), sizes,
+                        out_dtype=torch.float32)
+        assert max_rel_err(out, exact) <= 1e-2, max_rel_err(out, exact)
+        assert max_rel_err(out, exact) <= TOL_FP8
+        # unquantised bf16 activations on de-quantised weights: activation rounding noise
+        ref = ffn.gmm(a, fp8.dequantize_weight(wq, w_s), sizes)
+        noise = max_rel_err(out, ref)
+        print(f"[fp8] gmm vs unquantised-activation oracle: {noise:.4f}")
+        assert noise <= TOL_FP8_ACT, noise
+    finally:
+        gg.set_tile_variant(0)
+
+
+def test_fp8_experts_forward():
+    announce(test="fp8_experts_forward")
+    E, d, I, R = 4, 512, 768, 600
+    g = torch.Generator().manual_seed(3)
+    w13 = (torch.randn(E, d, 2 * I, generator=g) * 0.02).to(torch.bfloat16)
+    w2 = (torch.randn(E, I, d, generator=g) * 0.02).to(torch.bfloat16)
+    x = torch.randn(R, d, generator=g).to(torch.bfloat16)
+    sizes = ragged_sizes(E, R, seed=9)
+    layer = MoEExpertsFP8(w13.to(dev()), w2.to(dev()))
+    out = layer.forward(R, x.to(dev()), sizes.to(dev()))
+    same_points = fp8.moe_experts_forward_fp8(x, layer.w13_q.cpu(), layer.w13_scale.cpu(), layer.w2_q.cpu(),
+                                              layer.w2_scale.cpu(), sizes)
+    assert max_rel_err(out, same_points) <= TOL_FP8, max_rel_err(out, same_points)
+    dq13 = fp8.dequantize_weight(layer.w13_q.cpu(), layer.w13_scale.cpu())
+    dq2 = fp8.dequantize_weight(layer.w2_q.cpu(), layer.w2_scale.cpu())
+    ref = ffn.moe_experts_forward(x, dq13, dq2, sizes)
+    noise = max_rel_err(out, ref)
+    print(f"[fp8] FFN vs unquantised-activation oracle: {noise:.4f}")
+    assert noise <= TOL_FP8_ACT, noise
+
+
+def test_c5_full_size_sampled():
+    w = workloads.WORKLOADS["C5"]
+    announce(test="fp8_c5", T=w.T, d=w.d, I=w.I, E=w.E)
+    from disagmoe_amd.expert_layer import expert_layer_forward
+    ids, gates = workloads.make_routing(w)
+    x = workloads.make_activations(w).to(dev())
+    w13, w2 = workloads.make_weights(w, dev())
+    layer = MoEExpertsFP8(w13, w2)
+    del w13, w2
+    stages = {}
+    out = expert_layer_forward(layer, x, ids.to(dev()), gates.to(dev()), stages=stages)
+    torch.cuda.synchronize()
+    cnt = stages["batch_sizes"].cpu().tolist()
+    off = stages["offsets"].cpu().tolist()
+    xp, y = stages["permuted"], stages["expert_out"]
+    worst = noise = 0.0
+    for e in range(w.E):
+        pick = torch.tensor(sorted({off[e], off[e] + cnt[e] - 1, off[e] + cnt[e] // 2, off[e] + 17}), device=dev())
+        q13, s13 = layer.w13_q[e:e + 1].cpu(), layer.w13_scale[e:e + 1].cpu()
+        q2, s2 = layer.w2_q[e:e + 1].cpu(), layer.w2_scale[e:e + 1].cpu()
+        same_points = fp8.moe_experts_forward_fp8(xp[pick].cpu(), q13, s13, q2, s2, [pick.numel()])
+        worst = max(worst, max_rel_err(y[pick], same_points))
+        ref = ffn.moe_experts_forward(xp[pick].cpu(), fp8.dequantize_weight(q13, s13), fp8.dequantize_weight(q2, s2),
+                                      [pick.numel()])
+        noise = max(noise, max_rel_err(y[pick], ref))
+    print(f"[fp8] C5 FFN: same quantisation points {worst:.4f}, unquantised-activation oracle {noise:.4f}")
+    assert worst <= TOL_FP8, worst
+    assert noise <= TOL_FP8_ACT, noise
+    assert torch.isfinite(out.float()).all()

@@ -1,0 +1,146 @@
+"""Grouped GEMM / expert FFN parity against the fp32-accumulated oracle.
+
+Tolerance (stated by the task): max|out - ref| / max|ref| <= 1e-2 for bf16."""
+import pytest
+import torch
+
+from disagmoe_amd import workloads
+from disagmoe_amd.executor import ExpertsExecutor
+from disagmoe_amd.config import ModelConfig
+from disagmoe_amd.grouped_gemm import backend as gg
+from disagmoe_amd.models.experts import MoEExperts, MoEExpertsSerial
+from oracle import ffn
+from helpers import TOL_BF16, announce, dev, max_rel_err, ragged_sizes
+
+pytestmark = pytest.mark.gpu
+
+
+def _rand(shape, seed, std=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * std).to(torch.bfloat16)
+
+
+@pytest.fixture(autouse=True)
+def _default_tile():
+    gg.set_tile_variant(0)
+    yield
+    gg.set_tile_variant(0)
+
+
+def test_reference_gemm_case():
+    # tests/ops/test_gemm.py:4-36: E=8, two rows per expert, 1024x1024; gmm == gmm_with_arguments (twice)
+    announce(test="gmm_reference_case")
+    E, hs = 8, 1024
+    w1 = _rand((E, hs, hs), 1).to(dev())
+    x = _rand((2 * E, hs), 2).to(dev())
+    batch_sizes = torch.tensor([2] * E, dtype=torch.int64)
+    y = gg.gmm(x, w1, batch_sizes)
+    size, ptr = gg.get_arguments(E, dev())
+    workspace = torch.empty([size], dtype=torch.uint8, device=dev())
+    y2 = gg.gmm_with_arguments(x, w1, batch_sizes, workspace, ptr)
+    y3 = gg.gmm_with_arguments(x, w1, batch_sizes, workspace, ptr)
+    assert torch.equal(y, y2) and torch.equal(y, y3)
+    assert max_rel_err(y, ffn.gmm(x.cpu(), w1.cpu(), batch_sizes)) <= TOL_BF16
+
+
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("E,R,K,N", [(1, 300, 256, 256), (4, 1000, 128, 512), (8, 777, 320, 264), (3, 64, 72, 40),
+                                     (5, 1500, 512, 768)])
+@pytest.mark.parametrize("trans_b", [False, True])
+def test_gmm_ragged(variant, E, R, K, N, trans_b):
+    announce(test="gmm_ragged", variant=variant, E=E, R=R, K=K, N=N, trans_b=trans_b)
+    gg.set_tile_variant(variant)
+    sizes = ragged_sizes(E, R, seed=E * 1000 + R)
+    a = _rand((R, K), 3)
+    b = _rand((E, N, K) if trans_b else (E, K, N), 4, std=0.05)
+    ref = ffn.gmm(a, b, sizes, trans_b=trans_b)
+    out = gg.gmm(a.to(dev()), b.to(dev()), sizes.to(dev()), trans_b=trans_b)
+    assert out.shape == (R, N) and out.dtype == torch.bfloat16
+    assert max_rel_err(out, ref) <= TOL_BF16, max_rel_err(out, ref)
+
+
+def test_gmm_single_expert_equals_matmul_and_zero_sizes():
+    announce(test="gmm_special_cases")
+    a = _rand((513, 384), 5).to(dev())
+    b = _rand((1, 384, 520), 6, std=0.05).to(dev())
+    out = gg.gmm(a, b, torch.tensor([513]))
+    assert max_rel_err(out, (a.float() @ b[0].float())) <= TOL_BF16
+    # all experts empty: the output buffer is left untouched
+    c = torch.full((513, 520), 3.0, dtype=torch.bfloat16, device=dev())
+    b4 = _rand((4, 384, 520), 7, std=0.05).to(dev())
+    out = gg.gmm(a, b4, torch.zeros(4, dtype=torch.int64), c=c)
+    assert out.data_ptr() == c.data_ptr() and (c == 3.0).all()
+    # rows past sum(batch_sizes) are left untouched; host or device sizes give the same bits
+    c.fill_(3.0)
+    sizes = torch.tensor([100, 0, 50, 7])
+    gg.gmm(a, b4, sizes, c=c)
+    assert (c[157:] == 3.0).all()
+    ref = ffn.gmm(a.cpu()[:157], b4.cpu(), sizes)
+    assert max_rel_err(c[:157], ref) <= TOL_BF16
+    c2 = gg.gmm(a, b4, sizes.to(dev()))
+    assert torch.equal(c2[:157], c[:157])
+    # sizes that overrun the buffer are clamped, nothing past the last row is touched
+    guard = torch.full((600, 520), 5.0, dtype=torch.bfloat16, device=dev())
+    gg.gmm(a, b4, torch.tensor([400, 400, 400, 400]), c=guard)
+    assert (guard[513:] == 5.0).all()
+
+
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("trans_b", [False, True])
+def test_gmm_swiglu(variant, trans_b):
+    announce(test="gmm_swiglu", variant=variant, trans_b=trans_b)
+    gg.set_tile_variant(variant)
+    E, R, K, I = 6, 900, 256, 328
+    sizes = ragged_sizes(E, R, seed=17)
+    a = _rand((R, K), 8)
+    w13 = _rand((E, K, 2 * I), 9, std=0.08)
+    up = torch.zeros(R, 2 * I)
+    o = 0
+    for e, n in enumerate(sizes.tolist()):
+        up[o:o + n] = a[o:o + n].float() @ w13[e].float()
+        o += n
+    ref = torch.nn.functional.silu(up[:, :I]) * up[:, I:]
+    b = w13.transpose(1, 2).contiguous() if trans_b else w13
+    out = gg.gmm_swiglu(a.to(dev()), b.to(dev()), sizes, trans_b=trans_b)
+    assert out.shape == (R, I)
+    assert max_rel_err(out, ref) <= TOL_BF16, max_rel_err(out, ref)
+
+
+@pytest.mark.parametrize("E,d,I,R", [(8, 1024, 2816, 1024), (4, 512, 704, 300), (64, 256, 192, 2000)])
+def test_moe_experts_forward(E, d, I, R):
+    announce(test="moe_experts_forward", E=E, d=d, I=I, R=R)
+    layer = MoEExperts(d, I, E, init_std=0.02)
+    assert layer.w13_weight.shape == (E, d, 2 * I) and layer.w2_weight.shape == (E, I, d)
+    assert sorted(layer.state_dict().keys()) == ["w13_weight", "w2_weight"]
+    sizes = ragged_sizes(E, R, seed=E + R)
+    x = _rand((R, d), 10).to(dev())
+    out = layer.forward(R, x, sizes.to(dev()))
+    ref = ffn.moe_experts_forward(x.cpu(), layer.w13_weight.cpu(), layer.w2_weight.cpu(), sizes)
+    assert out.shape == (R, d)
+    assert max_rel_err(out, ref) <= TOL_BF16, max_rel_err(out, ref)
+    # the reference's unfused schedule (four roundings) agrees within the same tolerance
+    assert max_rel_err(layer.forward_unfused(R, x, sizes.to(dev())), ref) <= TOL_BF16
+    # static-buffer path (bs below max_batch_size) gives the same bits as the allocating path
+    small = MoEExperts(d, I, E, init_std=0.02, max_batch_size=R)
+    small.load_state_dict(layer.state_dict())
+    assert torch.equal(small.forward(R, x, sizes.to(dev())), out)
+
+
+def test_serial_experts_and_executor():
+    announce(test="serial_and_executor")
+    E, d, I, R = 4, 512, 768, 200
+    cfg = ModelConfig(hidden_size=d, num_layers=2, num_heads=8, num_kv_heads=8, num_experts=E, intermediate_size=I,
+                      layer_ids=[3, 7], top_k=2, max_batch_size_expert=64)
+    ex = ExpertsExecutor(cfg, init_std=0.02)
+    assert len(ex.operators) == 2 and isinstance(ex.operators[0], MoEExperts)
+    sizes = ragged_sizes(E, R, seed=1)
+    x = _rand((R, d), 11).to(dev())
+    out = ex.execute(7, R, x, sizes.to(dev()))
+    op = ex.operators[1]
+    ref = ffn.moe_experts_forward(x.cpu(), op.w13_weight.cpu(), op.w2_weight.cpu(), sizes)
+    assert max_rel_err(out, ref) <= TOL_BF16
+    serial = MoEExpertsSerial(d, I, E, init_std=0.02)
+    serial.load_state_dict(op.state_dict())
+    assert max_rel_err(serial.forward(R, x, sizes), ref) <= TOL_BF16
+    cfg.enable_grouped_gemm = False
+    assert isinstance(ExpertsExecutor(cfg, init_std=0.02).operators[0], MoEExpertsSerial)

@@ -102,10 +102,17 @@ __device__ __forceinline__ TileCoord decode_tile(long long q, int G, long long t
     }
     TileCoord t;
     t.e = lo;
+    // inside an expert: bands of up to kBand m-tiles; a band walks the n-tiles with its m-tiles innermost, so
+    // a weight tile is shared by the band's m-tiles and the band's A rows stay in L2 while it sweeps N
+    constexpr int kBand = 4;
     const int mt_e = s_tile_start[lo + 1] - s_tile_start[lo];
-    const int local = (int)(L - (long long)s_tile_start[lo] * n_tiles);
-    t.nt = local / mt_e;
-    const int mi = local - t.nt * mt_e;
+    int idx = (int)(L - (long long)s_tile_start[lo] * n_tiles);
+    const int full = mt_e / kBand;
+    int band = idx / (kBand * n_tiles), width = kBand;
+    if (band >= full) { band = full; width = mt_e - full * kBand; }
+    idx -= band * kBand * n_tiles;
+    t.nt = idx / width;
+    const int mi = band * kBand + (idx - t.nt * width);
     t.row0 = s_row_start[lo] + mi * BM;
     t.rows_e = s_row_start[lo + 1] - t.row0;
     return t;

@@ -92,7 +92,12 @@ void gmm_direct_kernel(const GmmArgs p) {
         // tile column slot (0..255) -> column of b; slots past the end read column n0 (never stored)
         auto b_col = [&](int slot) {
             const int rh = (SWIGLU && slot >= kDN / 2) ? slot - kDN / 2 : slot;
-            const int base = (SWIGLU && slot >= kDN / 2) ? n_out + n0 : n0;
+#ifdef DMOE_DBG_SAME_B
+            const int nb = 0;       // timing experiment: every n-tile reads the first weight tile (wrong results)
+#else
+            const int nb = n0;
+#endif
+            const int base = (SWIGLU && slot >= kDN / 2) ? n_out + nb : nb;
             return base + (rh < half_cols ? rh : 0);
         };
 
@@ -108,24 +113,30 @@ void gmm_direct_kernel(const GmmArgs p) {
         }
         if constexpr (!TRANS_B) b_off[0] = (uint32_t)kn_k * (uint32_t)p.N * 2 + (uint32_t)b_col(kn_chunk * 8) * 2;
 
-        auto issue_loads = [&](int s) {
+        // copy number c (0..7) of this wavefront for stage s: 0..3 are its A blocks, 4..7 its B blocks
+        auto issue_copy = [&](int s, int c) {
+#ifdef DMOE_DBG_NO_GLOAD
+            if (s >= kStages) return;   // timing experiment: no global traffic after the prologue (wrong results)
+#endif
+#ifdef DMOE_DBG_SKIP_A
+            if (s >= kStages && c < 4) return;
+#endif
+#ifdef DMOE_DBG_SKIP_B
+            if (s >= kStages && c >= 4) return;
+#endif
             const uint32_t lA = smem_addr + (s & (kStages - 1)) * kStage + wave * 1024;
-            const uint32_t lB = lA + kStageA;
-            const char *ga = a_base + (long long)s * (kDK * 2);
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-                copy_g2lds_16(ga + a_off[i], lA + i * 4096);
-            if constexpr (TRANS_B) {
-                const char *gb = b_exp + (long long)s * (kDK * 2);
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    copy_g2lds_16(gb + b_off[i], lB + i * 4096);
+            if (c < 4) {
+                copy_g2lds_16(a_base + (long long)s * (kDK * 2) + a_off[c], lA + c * 4096);
             } else {
-                const char *gb = b_exp + (long long)s * kDK * p.N * 2 + b_off[0];
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    copy_g2lds_16(gb + (long long)i * 8 * p.N * 2, lB + i * 4096);
+                const int i = c - 4;
+                const uint32_t lB = lA + kStageA + i * 4096;
+                if constexpr (TRANS_B) copy_g2lds_16(b_exp + (long long)s * (kDK * 2) + b_off[i], lB);
+                else copy_g2lds_16(b_exp + ((long long)s * kDK + i * 8) * p.N * 2 + b_off[0], lB);
             }
+        };
+        auto issue_loads = [&](int s) {
+#pragma unroll
+            for (int c = 0; c < kLoads; ++c) issue_copy(s, c);
         };
 
         // B operand rows / columns of this wavefront: fragment j covers 32 tile columns
@@ -143,17 +154,16 @@ void gmm_direct_kernel(const GmmArgs p) {
         }
 
         bf16x8 fa[2][4], fb[2][4];
-        auto load_frags = [&](int s, int ks, int slot) {
+        // operand read number r (0..7) of k-step ks of stage s into register set `slot`: 0..3 A, 4..7 B fragments
+        auto load_frag = [&](int s, int ks, int slot, int r) {
             const char *tA = smem + (s & (kStages - 1)) * kStage;
             const char *tB = tA + kStageA;
             const int c0 = ((ks * 2 + kgrp) ^ f_sw) << 4;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const u32x4 x = *(const u32x4 *)(tA + fa_base + i * 2048 + c0);
-                __builtin_memcpy(&fa[slot][i], &x, 16);
-            }
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
+            if (r < 4) {
+                const u32x4 x = *(const u32x4 *)(tA + fa_base + r * 2048 + c0);
+                __builtin_memcpy(&fa[slot][r], &x, 16);
+            } else {
+                const int j = r - 4;
                 if constexpr (TRANS_B) {
                     const u32x4 x = *(const u32x4 *)(tB + fb_off[j] + c0);
                     __builtin_memcpy(&fb[slot][j], &x, 16);
@@ -166,6 +176,10 @@ void gmm_direct_kernel(const GmmArgs p) {
                 }
             }
         };
+        auto load_frags = [&](int s, int ks, int slot) {
+#pragma unroll
+            for (int r = 0; r < 8; ++r) load_frag(s, ks, slot, r);
+        };
 
         f32x16 acc[4][4];
 #pragma unroll
@@ -174,12 +188,9 @@ void gmm_direct_kernel(const GmmArgs p) {
             for (int j = 0; j < 4; ++j)
 #pragma unroll
                 for (int x = 0; x < 16; ++x) acc[i][j][x] = 0.f;
-        auto mfma_all = [&](int slot) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[slot][i], fb[slot][j], acc[i][j], 0, 0, 0);
+        auto mfma_one = [&](int slot, int t) {
+            const int i = t >> 2, j = t & 3;
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[slot][i], fb[slot][j], acc[i][j], 0, 0, 0);
         };
 
         // ---- prologue: every LDS stage is free (the previous tile ended with a barrier after its last read) ----
@@ -192,30 +203,49 @@ void gmm_direct_kernel(const GmmArgs p) {
         __syncthreads();
         load_frags(0, 0, 0);
 
-        // One stage: k-step 0, then k-step 1 with the hand-over to stage s+1 behind its first MFMAs.
-        // kAhead = stages after s+1 whose copies are already in flight (they may still be when s+1 is opened).
-        auto run_stage = [&](int s, auto ahead_tag, auto next_tag) {
+        // One stage = 2 k-steps of 16 MFMAs.  A wavefront issues in order and an MFMA occupies the matrix
+        // pipe for 32 cycles, so the LDS reads and global -> LDS copies are slotted one per MFMA: they are
+        // issued in the shadow of the MFMA before them and the pipe never waits for the issue port.
+        //   k-step 0: MFMAs on register set 0; the 8 operand reads of k-step 1 go to set 1.
+        //   hand-over: this wavefront's share of stage s+1 has landed (vmcnt), barrier (everybody's has, and
+        //              every read of stage s is complete).
+        //   k-step 1: MFMAs on set 1; the 8 operand reads of stage s+1 go to set 0, then the 8 copies that
+        //              refill the LDS stage just drained with stage s+4.
+        // kAhead = stages after s+1 whose copies are already in flight when s+1 is opened.
+        auto run_stage = [&](int s, auto ahead_tag, auto next_tag, auto copy_tag) {
             constexpr int kAhead = decltype(ahead_tag)::value;
             constexpr bool kNext = decltype(next_tag)::value;
-            load_frags(s, 1, 1);
-            __builtin_amdgcn_sched_barrier(0);      // keep the operand reads ahead of the MFMAs that hide them
-            mfma_all(0);
-            __builtin_amdgcn_sched_barrier(0);      // the hand-over below stays behind these MFMAs
-            if constexpr (kNext) {
-                DMOE_WAIT_VMCNT(kAhead * kLoads);   // this wavefront's share of stage s+1 has landed ...
-                __syncthreads();                    // ... so has everybody else's; all reads of stage s are done
-                if (s + kStages < S) issue_loads(s + kStages);   // refill the stage just drained
-                load_frags(s + 1, 0, 0);
+            constexpr bool kCopy = decltype(copy_tag)::value;
+#pragma unroll
+            for (int t = 0; t < 16; ++t) {
+                mfma_one(0, t);
+                if (t < 8) load_frag(s, 1, 1, t);
                 __builtin_amdgcn_sched_barrier(0);
             }
-            mfma_all(1);
-            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (kNext) {
+                DMOE_WAIT_VMCNT(kAhead * kLoads);
+                __syncthreads();
+                __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int t = 0; t < 16; ++t) {
+                mfma_one(1, t);
+                if constexpr (kNext) {
+                    if (t < 8) load_frag(s + 1, 0, 0, t);
+                    else if constexpr (kCopy) issue_copy(s + kStages, t - 8);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
         };
+        typedef std::integral_constant<int, 2> two_t;
+        typedef std::integral_constant<int, 1> one_t;
+        typedef std::integral_constant<int, 0> zero_t;
         int s = 0;
-        for (; s + 3 < S; ++s) run_stage(s, std::integral_constant<int, 2>{}, std::true_type{});
-        if (s + 2 < S) { run_stage(s, std::integral_constant<int, 1>{}, std::true_type{}); ++s; }
-        if (s + 1 < S) { run_stage(s, std::integral_constant<int, 0>{}, std::true_type{}); ++s; }
-        run_stage(s, std::integral_constant<int, 0>{}, std::false_type{});
+        for (; s + kStages < S; ++s) run_stage(s, two_t{}, std::true_type{}, std::true_type{});
+        if (s + 3 < S) { run_stage(s, two_t{}, std::true_type{}, std::false_type{}); ++s; }
+        if (s + 2 < S) { run_stage(s, one_t{}, std::true_type{}, std::false_type{}); ++s; }
+        if (s + 1 < S) { run_stage(s, zero_t{}, std::true_type{}, std::false_type{}); ++s; }
+        run_stage(s, zero_t{}, std::false_type{}, std::false_type{});
         __syncthreads();   // the last stage has been read by everyone before the next tile refills LDS
 
         // ---- epilogue: accumulator (row, col) = ((x/4)*8 + (lane/32)*4 + x%4, lane%32) ----

@@ -20,7 +20,7 @@ ARCH = "gfx950"
 FLAGS = [
     f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option",
+    "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option", "-Wno-inline-asm",
 ]
 
 

@@ -17,6 +17,8 @@
 //     its way into LDS so that both MFMA operands are read K-contiguous;
 //   * each wavefront owns a TM x TN sub-tile as FM x FN accumulators of
 //     v_mfma_f32_32x32x16_bf16 (v_mfma_f32_32x32x64_f8f6f4 for fp8).
+#include <atomic>
+
 #include "gmm_common.h"
 
 namespace dmoe {
@@ -94,7 +96,16 @@ void gmm_kernel(const GmmArgs p) {
     const int fb_off = ((SWIGLU ? wn * (TN / 2) : wn * TN) + l31) * kRowBytes;
     const int fsw = swz(l31);
 
-    for (long long q = blockIdx.x; q < total; q += G) {
+    __shared__ long long s_item;
+    const int streams = (G % kXcds == 0) ? kXcds : 1;
+    unsigned int draw = 0;
+    if (tid == 0) draw = sched_draw(p.sched_slot, streams);
+    for (;;) {
+        if (tid == 0) s_item = sched_item(draw, streams);
+        __syncthreads();
+        const long long q = s_item;
+        if (q >= total) break;
+        if (tid == 0) draw = sched_draw(p.sched_slot, streams);   // next item; the round trip hides behind this tile
         const TileCoord tc = decode_tile<BM>(q, G, total, n_tiles, E, s_tile_start, s_row_start);
         const int e = tc.e, nt = tc.nt, row0 = tc.row0, rows_e = tc.rows_e;
         const int n0 = nt * BNO;                               // first output column
@@ -254,16 +265,21 @@ void gmm_kernel(const GmmArgs p) {
                 }
             }
         };
+        // row fragments of this wavefront that hold at least one valid row (a short last tile skips the rest)
+        int nfr = ((rows_e < BM ? rows_e : BM) - wm * TM + 31) / 32;
+        nfr = nfr < 0 ? 0 : (nfr > FM ? FM : nfr);
         auto mfma_all = [&](f32x16 (&acc)[FM][FN], int slot) {
 #pragma unroll
-            for (int i = 0; i < FM; ++i)
+            for (int i = 0; i < FM; ++i) {
+                if (i >= nfr) continue;
 #pragma unroll
                 for (int j = 0; j < FN; ++j) {
                     if constexpr (FP8)
-                        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[slot][i], fb[slot][j], acc[i][j], 0, 0, 0, 0, 0, 0);
+                        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[slot][j], fa[slot][i], acc[i][j], 0, 0, 0, 0, 0, 0);
                     else
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[slot][i], fb[slot][j], acc[i][j], 0, 0, 0);
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[slot][j], fa[slot][i], acc[i][j], 0, 0, 0);
                 }
+            }
         };
 
         f32x16 acc[FM][FN];
@@ -334,39 +350,54 @@ void gmm_kernel(const GmmArgs p) {
             if (grp == 0) __syncthreads();
         }
 
-        // ---- epilogue: accumulator (row, col) = ((x/4)*8 + (lane/32)*4 + x%4, lane%32) ----
-        uint16_t *cbase = (uint16_t *)p.c;
+        // ---- epilogue ----
+        // The MFMAs take the B fragment as their first operand, so an accumulator holds the tile transposed:
+        // lane l owns output row l % 32 of its fragment and, in element x, column (x/4)*8 + (l/32)*4 + x%4.
+        // Four consecutive columns per lane -> one 8-byte store; a row is valid or not per lane.
         constexpr int FNO = SWIGLU ? FN / 2 : FN;
 #pragma unroll
         for (int i = 0; i < FM; ++i) {
+            const int r = wm * TM + i * 32 + l31;
+            if (r >= rows_e) continue;
+            const int col_lane = n0 + (SWIGLU ? wn * (TN / 2) : wn * TN) + kgrp * 4;
+            uint16_t *crow = (uint16_t *)p.c + (long long)(row0 + r) * p.ldc + col_lane;
+            float sa = 1.f;
+            if (FP8) sa = p.a_scale[row0 + r];
 #pragma unroll
             for (int j = 0; j < FNO; ++j) {
-                const int ccol = n0 + (SWIGLU ? wn * (TN / 2) : wn * TN) + j * 32 + l31;
-                if (ccol >= n_out) continue;
-                float sb0 = 1.f, sb1 = 1.f;
-                if (FP8) {
-                    sb0 = p.b_scale[(long long)e * p.N + ccol];
-                    if (SWIGLU) sb1 = p.b_scale[(long long)e * p.N + n_out + ccol];
-                }
 #pragma unroll
-                for (int x = 0; x < 16; ++x) {
-                    const int r = wm * TM + i * 32 + (x >> 2) * 8 + kgrp * 4 + (x & 3);
-                    if (r >= rows_e) continue;
-                    float sa = 1.f;
-                    if (FP8) sa = p.a_scale[row0 + r];
-                    float v;
-                    if (SWIGLU) {
-                        const float g = acc[i][j][x] * (sa * sb0);
-                        const float up = acc[i][j + FN / 2][x] * (sa * sb1);
-                        v = g / (1.f + __expf(-g)) * up;
-                    } else {
-                        v = acc[i][j][x] * (sa * sb0);
+                for (int g = 0; g < 4; ++g) {
+                    const int col = col_lane + j * 32 + g * 8;
+                    if (col >= n_out) continue;                 // n_out % 8 == 0: four columns at once
+                    float sb0[4] = {1.f, 1.f, 1.f, 1.f}, sb1[4] = {1.f, 1.f, 1.f, 1.f};
+                    if (FP8) {
+                        const float4 t0 = *(const float4 *)(p.b_scale + (long long)e * p.N + col);
+                        sb0[0] = t0.x; sb0[1] = t0.y; sb0[2] = t0.z; sb0[3] = t0.w;
+                        if (SWIGLU) {
+                            const float4 t1 = *(const float4 *)(p.b_scale + (long long)e * p.N + n_out + col);
+                            sb1[0] = t1.x; sb1[1] = t1.y; sb1[2] = t1.z; sb1[3] = t1.w;
+                        }
                     }
-                    cbase[(long long)(row0 + r) * p.ldc + ccol] = f32_to_bf16(v);
+                    float v[4];
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) {
+                        if (SWIGLU) {
+                            const float gate = acc[i][j][g * 4 + x] * (sa * sb0[x]);
+                            const float up = acc[i][j + FN / 2][g * 4 + x] * (sa * sb1[x]);
+                            v[x] = gate / (1.f + __expf(-gate)) * up;
+                        } else {
+                            v[x] = acc[i][j][g * 4 + x] * (sa * sb0[x]);
+                        }
+                    }
+                    uint2 packed;
+                    packed.x = pack_bf16x2(v[0], v[1]);
+                    packed.y = pack_bf16x2(v[2], v[3]);
+                    *(uint2 *)(crow + j * 32 + g * 8) = packed;
                 }
             }
         }
     }
+    sched_finish(p.sched_slot);
 }
 
 template <int BM, int BN, int WM, int WN, bool TRANS_B, bool SWIGLU, bool FP8>
@@ -386,12 +417,19 @@ static int launch_one(const GmmArgs &args, hipStream_t stream) {
     long long grid = (long long)device_cus();
     if (m_tiles_max * n_tiles < grid) grid = m_tiles_max * n_tiles;
     if (grid < 1) grid = 1;
-    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NT), lds, stream, args);
+    GmmArgs launch_args = args;
+    launch_args.sched_slot = next_sched_slot();
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NT), lds, stream, launch_args);
     DMOE_LAUNCH_CHECK("gmm_kernel");
     return DMOE_OK;
 }
 
 static int g_variant = 0;  // tuning hook, see dmoe_gmm_tune
+
+int next_sched_slot() {
+    static std::atomic<unsigned int> counter{0};
+    return (int)(counter.fetch_add(1, std::memory_order_relaxed) % kSchedSlots);
+}
 
 template <bool TRANS_B, bool SWIGLU, bool FP8>
 static int launch_by_rows(const GmmArgs &args, hipStream_t stream) {

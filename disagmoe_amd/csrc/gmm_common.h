@@ -28,7 +28,46 @@ struct GmmArgs {
     int K;          // contraction length (elements)
     int N;          // columns of b per expert (2*I for the swiglu form)
     int ldc;        // columns of c (N, or I for the swiglu form)
+    int sched_slot; // entry of the work-counter ring used by this launch
 };
+
+// ---- work distribution ---------------------------------------------------------------------------
+// Tiles differ in cost (an expert's last m-tile may hold a few rows), so workgroups draw work items from
+// counters instead of striding over them.  There is one counter per XCD (workgroup id % 8): XCD x draws
+// j = 0, 1, 2, ... and works on item q = 8 j + x, which keeps the items that share operand tiles on one
+// L2 (see decode_tile) exactly as a static stride would, while a slow tile no longer holds up the tiles
+// queued behind it.  The counters of a launch live in one entry of a small ring in device memory; the
+// last workgroup to finish clears the entry, so no host-side reset or scratch argument is needed.
+// Launches that run concurrently must not share an entry: the host hands entries out round-robin.
+constexpr int kSchedSlots = 64;
+struct SchedSlot {
+    unsigned int next[kXcds];
+    unsigned int done;
+    unsigned int pad[7];
+};
+static __device__ SchedSlot g_sched[kSchedSlots];
+
+// Next work item of this workgroup (all threads get the same value), or -1 when its stream is exhausted.
+// `carry` holds the draw made ahead of time by thread 0 (see sched_draw).
+__device__ __forceinline__ unsigned int sched_draw(int slot, int streams) {
+    return atomicAdd(&g_sched[slot].next[streams == 1 ? 0 : (blockIdx.x % kXcds)], 1u);
+}
+__device__ __forceinline__ long long sched_item(unsigned int j, int streams) {
+    return streams == 1 ? (long long)j : (long long)j * kXcds + (blockIdx.x % kXcds);
+}
+// Called once per workgroup after its last draw; the last caller of the launch clears the entry.
+__device__ __forceinline__ void sched_finish(int slot) {
+    if (threadIdx.x == 0) {
+        __threadfence();
+        const unsigned int before = atomicAdd(&g_sched[slot].done, 1u);
+        if (before == gridDim.x - 1) {
+#pragma unroll
+            for (int i = 0; i < kXcds; ++i) g_sched[slot].next[i] = 0;
+            g_sched[slot].done = 0;
+            __threadfence();
+        }
+    }
+}
 
 // Prefix sums of rows and m-tiles over the experts, built by the first wavefront
 // into LDS tables of E + 1 entries.  Sizes are clamped so that the running row
@@ -81,9 +120,11 @@ struct TileCoord {
     int rows_e;   // rows of the expert from row0 on (>= 1; the tile holds min(rows_e, BM) of them)
 };
 
-// Work item q of workgroup-strided order -> tile.  Consecutive blocks of G/8 items go to the
-// workgroups of one XCD (workgroup id % 8); inside an expert the order is m-fastest, so the
-// m-tiles that share a weight tile run next to each other on one L2.
+// Work item q -> tile.  Items are cut in rounds of G (the grid size); inside a round, item q belongs to XCD
+// q % 8 and the XCD's items of the round are consecutive tiles.  Inside an expert the tiles are ordered in
+// bands of 4 m-tiles (a lone fifth, ninth, ... m-tile joins the band before it); a band walks the n-tiles
+// with its m-tiles innermost, so a weight tile is shared by the band's m-tiles on one L2 and the band's A
+// rows stay there while it sweeps N.
 template <int BM>
 __device__ __forceinline__ TileCoord decode_tile(long long q, int G, long long total, int n_tiles, int E,
                                                  const int *s_tile_start, const int *s_row_start) {
@@ -102,14 +143,17 @@ __device__ __forceinline__ TileCoord decode_tile(long long q, int G, long long t
     }
     TileCoord t;
     t.e = lo;
-    // inside an expert: bands of up to kBand m-tiles; a band walks the n-tiles with its m-tiles innermost, so
-    // a weight tile is shared by the band's m-tiles and the band's A rows stay in L2 while it sweeps N
     constexpr int kBand = 4;
     const int mt_e = s_tile_start[lo + 1] - s_tile_start[lo];
     int idx = (int)(L - (long long)s_tile_start[lo] * n_tiles);
-    const int full = mt_e / kBand;
+    int bands = mt_e / kBand;                       // full bands
+    const int rest = mt_e - bands * kBand;          // 0..3 m-tiles left over
     int band = idx / (kBand * n_tiles), width = kBand;
-    if (band >= full) { band = full; width = mt_e - full * kBand; }
+    if (rest == 1 && bands > 0) {                   // the lone m-tile rides with the last full band
+        if (band >= bands - 1) { band = bands - 1; width = kBand + 1; }
+    } else if (band >= bands) {
+        band = bands; width = rest;
+    }
     idx -= band * kBand * n_tiles;
     t.nt = idx / width;
     const int mi = band * kBand + (idx - t.nt * width);
@@ -118,6 +162,7 @@ __device__ __forceinline__ TileCoord decode_tile(long long q, int G, long long t
     return t;
 }
 
+int next_sched_slot();
 int launch_direct_bf16(const GmmArgs &args, bool trans_b, bool swiglu, hipStream_t stream);
 
 }  // namespace dmoe

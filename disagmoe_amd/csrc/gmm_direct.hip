@@ -83,7 +83,16 @@ void gmm_direct_kernel(const GmmArgs p) {
     const int f_sw = (l31 >> 2) & 3;
     const int g16 = lane >> 4, i16 = lane & 15;
 
-    for (long long q = blockIdx.x; q < total; q += G) {
+    __shared__ long long s_item;
+    const int streams = (G % kXcds == 0) ? kXcds : 1;
+    unsigned int draw = 0;
+    if (tid == 0) draw = sched_draw(p.sched_slot, streams);
+    for (;;) {
+        if (tid == 0) s_item = sched_item(draw, streams);
+        __syncthreads();
+        const long long q = s_item;
+        if (q >= total) break;
+        if (tid == 0) draw = sched_draw(p.sched_slot, streams);   // next item; the round trip hides behind this tile
         const TileCoord tc = decode_tile<kDM>(q, G, total, n_tiles, E, s_tile_start, s_row_start);
         const int e = tc.e, row0 = tc.row0, rows_e = tc.rows_e;
         const int n0 = tc.nt * BNO;
@@ -188,9 +197,13 @@ void gmm_direct_kernel(const GmmArgs p) {
             for (int j = 0; j < 4; ++j)
 #pragma unroll
                 for (int x = 0; x < 16; ++x) acc[i][j][x] = 0.f;
+        // row fragments of this wavefront that hold at least one valid row (a short last tile skips the rest)
+        int nfr = ((rows_e < kDM ? rows_e : kDM) - wm * 128 + 31) / 32;
+        nfr = nfr < 0 ? 0 : (nfr > 4 ? 4 : nfr);
         auto mfma_one = [&](int slot, int t) {
             const int i = t >> 2, j = t & 3;
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[slot][i], fb[slot][j], acc[i][j], 0, 0, 0);
+            if (i >= nfr) return;   // wave-uniform: a scalar branch around the MFMA
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[slot][j], fa[slot][i], acc[i][j], 0, 0, 0);
         };
 
         // ---- prologue: every LDS stage is free (the previous tile ended with a barrier after its last read) ----
@@ -248,31 +261,41 @@ void gmm_direct_kernel(const GmmArgs p) {
         run_stage(s, zero_t{}, std::false_type{}, std::false_type{});
         __syncthreads();   // the last stage has been read by everyone before the next tile refills LDS
 
-        // ---- epilogue: accumulator (row, col) = ((x/4)*8 + (lane/32)*4 + x%4, lane%32) ----
-        uint16_t *cbase = (uint16_t *)p.c;
+        // ---- epilogue ----
+        // The MFMAs take the B fragment as their first operand, so an accumulator holds the tile transposed:
+        // lane l owns output row l % 32 of its fragment and, in element x, column (x/4)*8 + (l/32)*4 + x%4.
+        // Four consecutive columns per lane -> one 8-byte store; a row is valid or not per lane.
         constexpr int FNO = SWIGLU ? 2 : 4;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
+            const int r = wm * 128 + i * 32 + l31;
+            if (r >= rows_e) continue;
+            uint16_t *crow = (uint16_t *)p.c + (long long)(row0 + r) * p.ldc + n0 + (SWIGLU ? wn * 64 : wn * 128) + kgrp * 4;
+            const int col_lane = n0 + (SWIGLU ? wn * 64 : wn * 128) + kgrp * 4;
 #pragma unroll
             for (int j = 0; j < FNO; ++j) {
-                const int ccol = n0 + (SWIGLU ? wn * 64 : wn * 128) + j * 32 + l31;
-                if (ccol >= n_out) continue;
 #pragma unroll
-                for (int x = 0; x < 16; ++x) {
-                    const int r = wm * 128 + i * 32 + (x >> 2) * 8 + kgrp * 4 + (x & 3);
-                    if (r >= rows_e) continue;
-                    float v;
-                    if (SWIGLU) {
-                        const float g = acc[i][j][x];
-                        v = g / (1.f + __expf(-g)) * acc[i][j + 2][x];
-                    } else {
-                        v = acc[i][j][x];
+                for (int g = 0; g < 4; ++g) {
+                    if (col_lane + j * 32 + g * 8 >= n_out) continue;   // n_out % 8 == 0: four columns at once
+                    float v[4];
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) {
+                        if (SWIGLU) {
+                            const float gate = acc[i][j][g * 4 + x];
+                            v[x] = gate / (1.f + __expf(-gate)) * acc[i][j + 2][g * 4 + x];
+                        } else {
+                            v[x] = acc[i][j][g * 4 + x];
+                        }
                     }
-                    cbase[(long long)(row0 + r) * p.ldc + ccol] = f32_to_bf16(v);
+                    uint2 packed;
+                    packed.x = pack_bf16x2(v[0], v[1]);
+                    packed.y = pack_bf16x2(v[2], v[3]);
+                    *(uint2 *)(crow + j * 32 + g * 8) = packed;
                 }
             }
         }
     }
+    sched_finish(p.sched_slot);
 }
 
 template <bool TRANS_B, bool SWIGLU>
@@ -291,7 +314,9 @@ static int launch_direct_one(const GmmArgs &args, hipStream_t stream) {
     long long grid = (long long)device_cus();
     if (m_tiles_max * n_tiles < grid) grid = m_tiles_max * n_tiles;
     if (grid < 1) grid = 1;
-    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), lds, stream, args);
+    GmmArgs launch_args = args;
+    launch_args.sched_slot = next_sched_slot();
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), lds, stream, launch_args);
     DMOE_LAUNCH_CHECK("gmm_direct_kernel");
     return DMOE_OK;
 }

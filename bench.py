@@ -24,9 +24,9 @@ PEAK_HBM_GBS = 8000.0
 PEAK_BF16_TFLOPS = 2500.0
 PEAK_FP8_TFLOPS = 5000.0
 
-# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc runs
-# (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known size); None until measured.
-MEASURED_TRAFFIC = {}
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc runs (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0,
+# the factors read off a 1 GiB copy in the same runs: profiles/expert_layer_c2_hbm_traffic.md); None = not measured.
+MEASURED_TRAFFIC = {"C2": 3.62e9}
 
 
 def _event_ms(fn, iters: int, warmup: int = 2):
@@ -58,20 +58,25 @@ def _cpu_baseline(w, x, ids, gates, layer, budget_s: float = 12.0):
     xc, idc, gc = x.cpu(), ids.cpu(), gates.cpu()
     n = min(w.T, 64)
     spent = 0.0
-    best = None
+    times = []
     while True:
         t0 = time.perf_counter()
         cpu_path.expert_layer(xc[:n], idc[:n], gc[:n], w13, w2)
         dt = time.perf_counter() - t0
         spent += dt
-        best = (n, dt)
-        if n >= w.T or spent + 2.2 * dt > budget_s:
+        if n < w.T and spent + 2.2 * dt <= budget_s:
+            n = min(w.T, n * 2)       # grow the sample while it is cheap
+            times = []
+            continue
+        times.append(dt)
+        if spent + dt > budget_s or len(times) >= 50:
             break
-        n = min(w.T, n * 2)
-    n, dt = best
+    times.sort()
+    dt = times[len(times) // 2]
     return {"value": n / dt, "unit": "tokens/s", "cores": cores, "kind": "port",
             "sample": f"first {n} of {w.T} tokens ({n * w.k} routed rows) through all {w.E} experts' full weights, "
-                      f"one pass, {dt:.2f} s; bf16 storage, torch CPU matmul (fp32 accumulate)"}
+                      f"median of {len(times)} passes, {dt:.2f} s each, {spent:.1f} s of CPU work in all; "
+                      f"bf16 storage, torch CPU matmul (fp32 accumulate)"}
 
 
 def main() -> int:
@@ -83,6 +88,8 @@ def main() -> int:
     ap.add_argument("--variant", type=int, default=0, help="grouped GEMM tile variant (tuning)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--kernel-iters", type=int, default=10)
+    ap.add_argument("--copy-probe-mib", type=int, default=0,
+                    help="also run a plain device copy of this many MiB (scales the FETCH_SIZE/WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the expert-worker path is built and measured on a single MI355X; "
@@ -125,6 +132,14 @@ def main() -> int:
         y = layer.forward(w.R, permuted, batch_sizes)
         return memory.combine_tokens(y, mappings, gates)
 
+    if args.copy_probe_mib > 0:
+        src = torch.empty(args.copy_probe_mib << 20, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -153,14 +168,16 @@ def main() -> int:
         q_ms, _ = _event_ms(lambda: gg.quantize_rows(permuted), it)
         stages["quant_rows"] = {"ms": q_ms}
         peak = PEAK_FP8_TFLOPS
-        kernel = "gmm_kernel<fp8, swiglu> (gate-up)"
+        kernel = "dmoe::gmm_kernel<.., swiglu, fp8> (gate-up projection with fused SiLU*mul)"
     else:
         h = gg.gmm_swiglu(permuted, layer.w13_weight, batch_sizes)
         up_ms, _ = _event_ms(lambda: gg.gmm_swiglu(permuted, layer.w13_weight, batch_sizes, c=h), it)
         y_buf = torch.empty((w.R, w.d), dtype=torch.bfloat16, device=dev)
         down_ms, _ = _event_ms(lambda: gg.gmm(h, layer.w2_weight, batch_sizes, c=y_buf), it)
         peak = PEAK_BF16_TFLOPS
-        kernel = "gmm_kernel<bf16, swiglu> (gate-up)"
+        big = w.R // w.E > 160 and w.d % 32 == 0
+        kernel = ("dmoe::gmm_direct_kernel<false, true>" if big else "dmoe::gmm_kernel<.., swiglu, bf16>") + \
+            " (gate-up projection with fused SiLU*mul)"
     up_flops = 2.0 * w.R * w.d * 2 * w.I
     down_flops = 2.0 * w.R * w.I * w.d
     stages["gemm_gate_up"] = {"ms": up_ms, "TFLOP/s": up_flops / up_ms / 1e9, "frac_mfma": up_flops / up_ms / 1e9 / peak}

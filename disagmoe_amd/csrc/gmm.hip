@@ -384,7 +384,7 @@ void gmm_kernel(const GmmArgs p) {
                         if (SWIGLU) {
                             const float gate = acc[i][j][g * 4 + x] * (sa * sb0[x]);
                             const float up = acc[i][j + FN / 2][g * 4 + x] * (sa * sb1[x]);
-                            v[x] = gate / (1.f + __expf(-gate)) * up;
+                            v[x] = silu_mul(gate, up);
                         } else {
                             v[x] = acc[i][j][g * 4 + x] * (sa * sb0[x]);
                         }
@@ -425,6 +425,9 @@ static int launch_one(const GmmArgs &args, hipStream_t stream) {
 }
 
 static int g_variant = 0;  // tuning hook, see dmoe_gmm_tune
+
+static int g_debug_mode = 0;
+int debug_mode() { return g_debug_mode; }
 
 int next_sched_slot() {
     static std::atomic<unsigned int> counter{0};
@@ -470,6 +473,9 @@ static int check_gmm(const char *who, const void *a, const void *b, const void *
 using namespace dmoe;
 
 extern "C" int dmoe_gmm_tune(int variant) {
+#ifdef DMOE_DEBUG_HOOKS
+    if (variant >= 100) { g_debug_mode = variant - 100; return DMOE_OK; }
+#endif
     DMOE_REQUIRE(variant >= 0 && variant <= 4, DMOE_ERR_ARG, "dmoe_gmm_tune: variant %d outside [0, 4]", variant);
     g_variant = variant;
     return DMOE_OK;

@@ -85,34 +85,28 @@ void gmm_direct_kernel(const GmmArgs p) {
 
     __shared__ long long s_item;
     const int streams = (G % kXcds == 0) ? kXcds : 1;
-    unsigned int draw = 0;
-    if (tid == 0) draw = sched_draw(p.sched_slot, streams);
-    for (;;) {
-        if (tid == 0) s_item = sched_item(draw, streams);
-        __syncthreads();
-        const long long q = s_item;
-        if (q >= total) break;
-        if (tid == 0) draw = sched_draw(p.sched_slot, streams);   // next item; the round trip hides behind this tile
-        const TileCoord tc = decode_tile<kDM>(q, G, total, n_tiles, E, s_tile_start, s_row_start);
-        const int e = tc.e, row0 = tc.row0, rows_e = tc.rows_e;
-        const int n0 = tc.nt * BNO;
-        const int half_cols = n_out - n0;                      // valid columns from n0 on
 
-        // tile column slot (0..255) -> column of b; slots past the end read column n0 (never stored)
-        auto b_col = [&](int slot) {
-            const int rh = (SWIGLU && slot >= kDN / 2) ? slot - kDN / 2 : slot;
-#ifdef DMOE_DBG_SAME_B
-            const int nb = 0;       // timing experiment: every n-tile reads the first weight tile (wrong results)
+    // ---- state of the tile whose copies are being issued (set by open_tile) ----
+    int e = 0, row0 = 0, rows_e = 0, n0 = 0;
+    const char *a_base = nullptr, *b_exp = nullptr;
+    uint32_t a_off[4], b_off[4];
+
+    // tile column slot (0..255) -> column of b; slots past the end read the first column (never stored)
+    auto b_col = [&](int slot) {
+        const int rh = (SWIGLU && slot >= kDN / 2) ? slot - kDN / 2 : slot;
+#ifdef DMOE_DEBUG_HOOKS
+        const int nb = p.dbg == 4 ? 0 : n0;   // timing experiment 4: every n-tile reads the first weight tile
 #else
-            const int nb = n0;
+        const int nb = n0;
 #endif
-            const int base = (SWIGLU && slot >= kDN / 2) ? n_out + nb : nb;
-            return base + (rh < half_cols ? rh : 0);
-        };
-
-        const char *a_base = p.a + (long long)row0 * pitch;
-        const char *b_exp = p.b + (long long)e * p.K * p.N * 2;
-        uint32_t a_off[4], b_off[4];
+        const int base = (SWIGLU && slot >= kDN / 2) ? n_out + nb : nb;
+        return base + (rh < n_out - n0 ? rh : 0);
+    };
+    auto open_tile = [&](long long q) {
+        const TileCoord tc = decode_tile<kDM>(q, G, total, n_tiles, E, s_tile_start, s_row_start);
+        e = tc.e; row0 = tc.row0; rows_e = tc.rows_e; n0 = tc.nt * BNO;
+        a_base = p.a + (long long)row0 * pitch;
+        b_exp = p.b + (long long)e * p.K * p.N * 2;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             int r = (i * 4 + wave) * 16 + kc_row;
@@ -121,74 +115,90 @@ void gmm_direct_kernel(const GmmArgs p) {
             if constexpr (TRANS_B) b_off[i] = (uint32_t)b_col((i * 4 + wave) * 16 + kc_row) * pitch + kc_chunk * 16;
         }
         if constexpr (!TRANS_B) b_off[0] = (uint32_t)kn_k * (uint32_t)p.N * 2 + (uint32_t)b_col(kn_chunk * 8) * 2;
+    };
 
-        // copy number c (0..7) of this wavefront for stage s: 0..3 are its A blocks, 4..7 its B blocks
-        auto issue_copy = [&](int s, int c) {
-#ifdef DMOE_DBG_NO_GLOAD
-            if (s >= kStages) return;   // timing experiment: no global traffic after the prologue (wrong results)
+    // copy number c (0..7) of this wavefront for stage s: 0..3 are its A blocks, 4..7 its B blocks
+    auto issue_copy = [&](int s, int c) {
+#ifdef DMOE_DEBUG_HOOKS
+        // timing experiments (wrong results): 1 = no copies after the prologue, 2 = no A copies, 3 = no B copies
+        if (s >= kStages && (p.dbg == 1 || (p.dbg == 2 && c < 4) || (p.dbg == 3 && c >= 4))) return;
 #endif
-#ifdef DMOE_DBG_SKIP_A
-            if (s >= kStages && c < 4) return;
-#endif
-#ifdef DMOE_DBG_SKIP_B
-            if (s >= kStages && c >= 4) return;
-#endif
-            const uint32_t lA = smem_addr + (s & (kStages - 1)) * kStage + wave * 1024;
-            if (c < 4) {
-                copy_g2lds_16(a_base + (long long)s * (kDK * 2) + a_off[c], lA + c * 4096);
-            } else {
-                const int i = c - 4;
-                const uint32_t lB = lA + kStageA + i * 4096;
-                if constexpr (TRANS_B) copy_g2lds_16(b_exp + (long long)s * (kDK * 2) + b_off[i], lB);
-                else copy_g2lds_16(b_exp + ((long long)s * kDK + i * 8) * p.N * 2 + b_off[0], lB);
-            }
-        };
-        auto issue_loads = [&](int s) {
+        const uint32_t lA = smem_addr + (s & (kStages - 1)) * kStage + wave * 1024;
+        if (c < 4) {
+            copy_g2lds_16(a_base + (long long)s * (kDK * 2) + a_off[c], lA + c * 4096);
+        } else {
+            const int i = c - 4;
+            const uint32_t lB = lA + kStageA + i * 4096;
+            if constexpr (TRANS_B) copy_g2lds_16(b_exp + (long long)s * (kDK * 2) + b_off[i], lB);
+            else copy_g2lds_16(b_exp + ((long long)s * kDK + i * 8) * p.N * 2 + b_off[0], lB);
+        }
+    };
+    const int pre = S < kStages ? S : kStages;      // stages whose copies are issued ahead of the tile's first MFMA
+    auto issue_prologue = [&]() {
+        for (int s = 0; s < pre; ++s) {
 #pragma unroll
             for (int c = 0; c < kLoads; ++c) issue_copy(s, c);
-        };
+        }
+    };
 
-        // B operand rows / columns of this wavefront: fragment j covers 32 tile columns
-        int fb_off[4];
+    // B operand rows / columns of this wavefront: fragment j covers 32 tile columns
+    int fb_off[4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int slot0 = SWIGLU ? ((j < 2) ? wn * 64 + j * 32 : kDN / 2 + wn * 64 + (j - 2) * 32) : wn * 128 + j * 32;
+    for (int j = 0; j < 4; ++j) {
+        const int slot0 = SWIGLU ? ((j < 2) ? wn * 64 + j * 32 : kDN / 2 + wn * 64 + (j - 2) * 32) : wn * 128 + j * 32;
+        if constexpr (TRANS_B) {
+            fb_off[j] = (slot0 + l31) * 64;
+        } else {
+            const int col = slot0 + (g16 & 1) * 16 + 4 * (i16 & 3);          // tile column of this lane's 4 values
+            const int chunk = (col >> 3) ^ (((i16 >> 2) & 3) << 2);
+            fb_off[j] = ((kgrp * 8) + (i16 >> 2)) * 512 + chunk * 16 + (col & 7) * 2;
+        }
+    }
+
+    bf16x8 fa[2][4], fb[2][4];
+    // operand read number r (0..7) of k-step ks of stage s into register set `slot`: 0..3 A, 4..7 B fragments
+    auto load_frag = [&](int s, int ks, int slot, int r) {
+        const char *tA = smem + (s & (kStages - 1)) * kStage;
+        const char *tB = tA + kStageA;
+        const int c0 = ((ks * 2 + kgrp) ^ f_sw) << 4;
+        if (r < 4) {
+            const u32x4 x = *(const u32x4 *)(tA + fa_base + r * 2048 + c0);
+            __builtin_memcpy(&fa[slot][r], &x, 16);
+        } else {
+            const int j = r - 4;
             if constexpr (TRANS_B) {
-                fb_off[j] = (slot0 + l31) * 64;
+                const u32x4 x = *(const u32x4 *)(tB + fb_off[j] + c0);
+                __builtin_memcpy(&fb[slot][j], &x, 16);
             } else {
-                const int col = slot0 + (g16 & 1) * 16 + 4 * (i16 & 3);          // tile column of this lane's 4 values
-                const int chunk = (col >> 3) ^ (((i16 >> 2) & 3) << 2);
-                fb_off[j] = ((kgrp * 8) + (i16 >> 2)) * 512 + chunk * 16 + (col & 7) * 2;
+                const char *src = tB + fb_off[j] + ks * (16 * 512);
+                const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)DMOE_LDS_PTR(src));
+                const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)DMOE_LDS_PTR(src + 4 * 512));
+                const s16x8 v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                __builtin_memcpy(&fb[slot][j], &v, 16);
             }
         }
+    };
 
-        bf16x8 fa[2][4], fb[2][4];
-        // operand read number r (0..7) of k-step ks of stage s into register set `slot`: 0..3 A, 4..7 B fragments
-        auto load_frag = [&](int s, int ks, int slot, int r) {
-            const char *tA = smem + (s & (kStages - 1)) * kStage;
-            const char *tB = tA + kStageA;
-            const int c0 = ((ks * 2 + kgrp) ^ f_sw) << 4;
-            if (r < 4) {
-                const u32x4 x = *(const u32x4 *)(tA + fa_base + r * 2048 + c0);
-                __builtin_memcpy(&fa[slot][r], &x, 16);
-            } else {
-                const int j = r - 4;
-                if constexpr (TRANS_B) {
-                    const u32x4 x = *(const u32x4 *)(tB + fb_off[j] + c0);
-                    __builtin_memcpy(&fb[slot][j], &x, 16);
-                } else {
-                    const char *src = tB + fb_off[j] + ks * (16 * 512);
-                    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)DMOE_LDS_PTR(src));
-                    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)DMOE_LDS_PTR(src + 4 * 512));
-                    const s16x8 v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                    __builtin_memcpy(&fb[slot][j], &v, 16);
-                }
-            }
-        };
-        auto load_frags = [&](int s, int ks, int slot) {
-#pragma unroll
-            for (int r = 0; r < 8; ++r) load_frag(s, ks, slot, r);
-        };
+    // ---- first work item ----
+    unsigned int draw = 0;
+    if (tid == 0) {
+        draw = sched_draw(p.sched_slot, streams);
+        s_item = sched_item(draw, streams);
+        draw = sched_draw(p.sched_slot, streams);   // always one draw ahead: its round trip hides behind a tile
+    }
+    __syncthreads();
+    long long q = s_item;
+    if (q < total) {
+        open_tile(q);
+        issue_prologue();
+    }
+
+    while (q < total) {
+        // results of this tile go here after the next tile's copies have been issued
+        const int cur_row0 = row0, cur_rows_e = rows_e, cur_n0 = n0;
+        // row fragments of this wavefront that hold at least one valid row (a short last tile skips the rest)
+        int nfr = ((rows_e < kDM ? rows_e : kDM) - wm * 128 + 31) / 32;
+        nfr = nfr < 0 ? 0 : (nfr > 4 ? 4 : nfr);
 
         f32x16 acc[4][4];
 #pragma unroll
@@ -197,24 +207,21 @@ void gmm_direct_kernel(const GmmArgs p) {
             for (int j = 0; j < 4; ++j)
 #pragma unroll
                 for (int x = 0; x < 16; ++x) acc[i][j][x] = 0.f;
-        // row fragments of this wavefront that hold at least one valid row (a short last tile skips the rest)
-        int nfr = ((rows_e < kDM ? rows_e : kDM) - wm * 128 + 31) / 32;
-        nfr = nfr < 0 ? 0 : (nfr > 4 ? 4 : nfr);
         auto mfma_one = [&](int slot, int t) {
             const int i = t >> 2, j = t & 3;
             if (i >= nfr) return;   // wave-uniform: a scalar branch around the MFMA
             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[slot][j], fa[slot][i], acc[i][j], 0, 0, 0);
         };
 
-        // ---- prologue: every LDS stage is free (the previous tile ended with a barrier after its last read) ----
-        const int pre = S < kStages ? S : kStages;
-        for (int s = 0; s < pre; ++s) issue_loads(s);
+        // stage 0 of this tile has landed (its other prologue stages, and stores of the previous tile's
+        // epilogue that were issued after them, may still be in flight: waiting for fewer is only stricter)
         if (pre == 4) DMOE_WAIT_VMCNT(3 * kLoads);
         else if (pre == 3) DMOE_WAIT_VMCNT(2 * kLoads);
         else if (pre == 2) DMOE_WAIT_VMCNT(kLoads);
         else DMOE_WAIT_VMCNT(0);
         __syncthreads();
-        load_frags(0, 0, 0);
+#pragma unroll
+        for (int r = 0; r < 8; ++r) load_frag(0, 0, 0, r);
 
         // One stage = 2 k-steps of 16 MFMAs.  A wavefront issues in order and an MFMA occupies the matrix
         // pipe for 32 cycles, so the LDS reads and global -> LDS copies are slotted one per MFMA: they are
@@ -259,41 +266,71 @@ void gmm_direct_kernel(const GmmArgs p) {
         if (s + 2 < S) { run_stage(s, one_t{}, std::true_type{}, std::false_type{}); ++s; }
         if (s + 1 < S) { run_stage(s, zero_t{}, std::true_type{}, std::false_type{}); ++s; }
         run_stage(s, zero_t{}, std::false_type{}, std::false_type{});
-        __syncthreads();   // the last stage has been read by everyone before the next tile refills LDS
 
-        // ---- epilogue ----
-        // The MFMAs take the B fragment as their first operand, so an accumulator holds the tile transposed:
-        // lane l owns output row l % 32 of its fragment and, in element x, column (x/4)*8 + (l/32)*4 + x%4.
-        // Four consecutive columns per lane -> one 8-byte store; a row is valid or not per lane.
-        constexpr int FNO = SWIGLU ? 2 : 4;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int r = wm * 128 + i * 32 + l31;
-            if (r >= rows_e) continue;
-            uint16_t *crow = (uint16_t *)p.c + (long long)(row0 + r) * p.ldc + n0 + (SWIGLU ? wn * 64 : wn * 128) + kgrp * 4;
-            const int col_lane = n0 + (SWIGLU ? wn * 64 : wn * 128) + kgrp * 4;
-#pragma unroll
-            for (int j = 0; j < FNO; ++j) {
-#pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    if (col_lane + j * 32 + g * 8 >= n_out) continue;   // n_out % 8 == 0: four columns at once
-                    float v[4];
-#pragma unroll
-                    for (int x = 0; x < 4; ++x) {
-                        if (SWIGLU) {
-                            const float gate = acc[i][j][g * 4 + x];
-                            v[x] = gate / (1.f + __expf(-gate)) * acc[i][j + 2][g * 4 + x];
-                        } else {
-                            v[x] = acc[i][j][g * 4 + x];
+        auto next_item = [&]() {
+            // ---- next work item and its first copies ----
+            if (tid == 0) s_item = sched_item(draw, streams);
+            __syncthreads();   // also: the last stage has been read by everyone, LDS may be refilled
+            q = s_item;
+            if (q < total) {
+                if (tid == 0) draw = sched_draw(p.sched_slot, streams);
+                open_tile(q);
+                issue_prologue();
+            }
+        };
+        auto epilogue = [&]() {
+            // ---- epilogue of the finished tile ----
+            // The MFMAs take the B fragment as their first operand, so an accumulator holds the tile transposed:
+            // lane l owns output row l % 32 of its fragment and, in element x, column (x/4)*8 + (l/32)*4 + x%4.
+            // Four consecutive columns per lane -> one 8-byte store; a row is valid or not per lane.
+            constexpr int FNO = SWIGLU ? 2 : 4;
+    #pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int r = wm * 128 + i * 32 + l31;
+                if (r >= cur_rows_e) continue;
+                const int col_lane = cur_n0 + (SWIGLU ? wn * 64 : wn * 128) + kgrp * 4;
+                uint16_t *crow = (uint16_t *)p.c + (long long)(cur_row0 + r) * p.ldc + col_lane;
+    #pragma unroll
+                for (int j = 0; j < FNO; ++j) {
+    #pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        if (col_lane + j * 32 + g * 8 >= n_out) continue;   // n_out % 8 == 0: four columns at once
+                        float v[4];
+    #pragma unroll
+                        for (int x = 0; x < 4; ++x) {
+                            if (SWIGLU) {
+                                const float gate = acc[i][j][g * 4 + x];
+                                v[x] = silu_mul(gate, acc[i][j + 2][g * 4 + x]);
+                            } else {
+                                v[x] = acc[i][j][g * 4 + x];
+                            }
                         }
+                        uint2 packed;
+                        packed.x = pack_bf16x2(v[0], v[1]);
+                        packed.y = pack_bf16x2(v[2], v[3]);
+#ifdef DMOE_DEBUG_HOOKS
+                        if (p.dbg == 7) {   // timing experiment: same bytes, fully coalesced addresses (wrong results)
+                            uint2 *lin = (uint2 *)((uint16_t *)p.c + (long long)cur_row0 * p.ldc) + ((wave * 64 + (i * 16 + j * 4 + g)) * 64 + lane);
+                            *lin = packed;
+                            continue;
+                        }
+#endif
+                        *(uint2 *)(crow + j * 32 + g * 8) = packed;
                     }
-                    uint2 packed;
-                    packed.x = pack_bf16x2(v[0], v[1]);
-                    packed.y = pack_bf16x2(v[2], v[3]);
-                    *(uint2 *)(crow + j * 32 + g * 8) = packed;
                 }
             }
-        }
+    
+        };
+#ifdef DMOE_DEBUG_HOOKS
+        // timing experiments: 5 = the next tile's first copies go out before the results are stored; 6 = results not stored
+        if (p.dbg == 5) { next_item(); epilogue(); }
+        else if (p.dbg == 6) { next_item(); }
+        else { epilogue(); next_item(); }
+#else
+        // stores first: they are then older than the next tile's copies and never hold up a vmcnt wait of its pipeline
+        epilogue();
+        next_item();
+#endif
     }
     sched_finish(p.sched_slot);
 }
@@ -316,6 +353,7 @@ static int launch_direct_one(const GmmArgs &args, hipStream_t stream) {
     if (grid < 1) grid = 1;
     GmmArgs launch_args = args;
     launch_args.sched_slot = next_sched_slot();
+    launch_args.dbg = debug_mode();
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), lds, stream, launch_args);
     DMOE_LAUNCH_CHECK("gmm_direct_kernel");
     return DMOE_OK;

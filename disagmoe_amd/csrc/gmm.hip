@@ -445,13 +445,14 @@ static int launch_by_rows(const GmmArgs &args, hipStream_t stream) {
         case 4: return launch_one<256, 256, 2, 4, TRANS_B, SWIGLU, FP8>(args, stream);
         default: break;
     }
-    if (avg <= 64) return launch_one<64, 256, 1, 4, TRANS_B, SWIGLU, FP8>(args, stream);
-    if (avg <= 160) return launch_one<128, 256, 1, 4, TRANS_B, SWIGLU, FP8>(args, stream);
+    const int tile_rows = avg <= 64 ? 64 : (avg <= 160 ? 128 : 256);
     if constexpr (!FP8) {
         // global -> LDS direct path: whole stages of 32 k, 32-bit offsets inside one expert's weights
         if (args.K % 32 == 0 && (long long)args.K * args.N * 2 < (1ll << 32))
-            return launch_direct_bf16(args, TRANS_B, SWIGLU, stream);
+            return launch_direct_bf16(args, tile_rows, TRANS_B, SWIGLU, stream);
     }
+    if (tile_rows == 64) return launch_one<64, 256, 1, 4, TRANS_B, SWIGLU, FP8>(args, stream);
+    if (tile_rows == 128) return launch_one<128, 256, 1, 4, TRANS_B, SWIGLU, FP8>(args, stream);
     return launch_one<256, 256, 2, 4, TRANS_B, SWIGLU, FP8>(args, stream);
 }
 

@@ -63,9 +63,11 @@ __device__ __forceinline__ void sched_finish(int slot) {
         __threadfence();
         const unsigned int before = atomicAdd(&g_sched[slot].done, 1u);
         if (before == gridDim.x - 1) {
+            // cleared with the same kind of operation the counters are advanced with, so that the clear is
+            // seen wherever the next launch's draws are performed
 #pragma unroll
-            for (int i = 0; i < kXcds; ++i) g_sched[slot].next[i] = 0;
-            g_sched[slot].done = 0;
+            for (int i = 0; i < kXcds; ++i) atomicExch(&g_sched[slot].next[i], 0u);
+            atomicExch(&g_sched[slot].done, 0u);
             __threadfence();
         }
     }
@@ -165,6 +167,6 @@ __device__ __forceinline__ TileCoord decode_tile(long long q, int G, long long t
 }
 
 int next_sched_slot();
-int launch_direct_bf16(const GmmArgs &args, bool trans_b, bool swiglu, hipStream_t stream);
+int launch_direct_bf16(const GmmArgs &args, int tile_rows, bool trans_b, bool swiglu, hipStream_t stream);
 
 }  // namespace dmoe

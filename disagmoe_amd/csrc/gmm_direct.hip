@@ -1,10 +1,11 @@
-// bf16 grouped GEMM, 256x256 tiles, for row counts that fill them: the CDNA4 data path.
+// bf16 grouped GEMM on the CDNA4 data path: tiles of 256, 128 or 64 rows by 256 columns.
 //
 //   * A and B tiles go global -> LDS directly (global_load_lds_dwordx4: each lane
 //     fetches 16 bytes, the wavefront fills 1 KiB of LDS), no staging registers,
 //     no LDS store instructions;
-//   * K is cut in stages of 32; four stages of 32 KiB live in LDS, so a load is
-//     issued three stages (about 3000 MFMA cycles) before its data is needed;
+//   * K is cut in stages of 32; 4 stages of 32 KiB (256-row tile), 5 of 24 KiB (128) or 6 of 20 KiB (64) live
+//     in LDS, so a copy is issued 3 to 5 stages before its data is needed (small tiles stream weights from
+//     HBM and need the depth);
 //   * the LDS images are permuted on the way in (the lane picks WHICH 16 bytes of
 //     the row it fetches) so that the operand reads are bank-conflict free:
 //       - K-contiguous operands ([rows][32 k] = 64 B rows): chunk ^ ((row >> 2) & 3),
@@ -12,9 +13,9 @@
 //       - B in the [K, N] layout is kept [k][256 n] (512 B rows): chunk ^ ((k & 3) << 2),
 //         read with ds_read_b64_tr_b16, which transposes 4 k x 16 n inside 16 lanes
 //         and hands every lane 4 consecutive k of its column - the MFMA B operand;
-//   * 4 wavefronts, one per SIMD, each owns 128x128 of the tile as 4x4
-//     v_mfma_f32_32x32x16_bf16 accumulators; operands are double buffered in
-//     registers one k-step ahead; one workgroup barrier per stage.
+//   * 4 wavefronts, one per SIMD; a wavefront owns 128x128 (256-row tile), 64x128 (128) or 64x64 (64) of
+//     the tile as 32x32 v_mfma_f32_32x32x16_bf16 accumulators; operands are double buffered in registers one
+//     k-step ahead; one workgroup barrier per stage.
 #include "gmm_common.h"
 
 namespace dmoe {
@@ -33,21 +34,30 @@ __device__ __forceinline__ void copy_g2lds_16(const char *gptr, uint32_t lds) {
 }
 __device__ __forceinline__ uint32_t lds_addr(const void *p) { return (uint32_t)(uintptr_t)DMOE_LDS_PTR(p); }
 
-constexpr int kDM = 256, kDN = 256;        // tile
+constexpr int kDN = 256;                   // tile columns
 constexpr int kDK = 32;                    // k per stage
-constexpr int kStages = 4;
-constexpr int kStageA = kDM * kDK * 2;     // 16 KiB
-constexpr int kStageB = kDN * kDK * 2;     // 16 KiB
-constexpr int kStage = kStageA + kStageB;
-constexpr int kLoads = 8;                  // global_load_lds per wavefront per stage (4 A + 4 B)
+constexpr int kStageB = kDN * kDK * 2;     // 16 KiB of B per stage
 
 // s_waitcnt with only vmcnt set (gfx9 encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14)
 #define DMOE_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (7 << 4) | (15 << 8) | (((n) >> 4) << 14))
 
-template <bool TRANS_B, bool SWIGLU>
+template <int kDM, int WM, bool TRANS_B, bool SWIGLU>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
 void gmm_direct_kernel(const GmmArgs p) {
+    constexpr int WN = 4 / WM;                           // wavefronts along N
+    constexpr int TM = kDM / WM, TN = kDN / WN;          // wave tile
+    constexpr int FM = TM / 32, FN = TN / 32;            // 32x32 accumulators per wavefront
+    constexpr int NM = FM * FN;                          // MFMAs per k-step
+    constexpr int NR = FM + FN;                          // operand reads per k-step (a B read = 2 transposing reads)
+    constexpr int CA = kDM / 64;                         // A copies (16 rows each) per wavefront per stage
+    constexpr int kLoads = CA + 4;                       // copies per wavefront per stage
+    constexpr int kStageA = kDM * kDK * 2;
+    constexpr int kStage = kStageA + kStageB;
+    constexpr int kStages = kDM == 256 ? 4 : (kDM == 128 ? 5 : 6);
     constexpr int BNO = SWIGLU ? kDN / 2 : kDN;
+    static_assert(kDM == 64 || kDM == 128 || kDM == 256, "tile rows");
+    static_assert(WM * WN == 4 && FM >= 1 && FN >= 2 && NR <= NM, "wave layout");
+    static_assert((kStages - 1) * kLoads <= 63, "vmcnt is a 6-bit counter");
     extern __shared__ __attribute__((aligned(16))) char smem[];
     __shared__ int s_tile_start[kMaxGroups + 1];
     __shared__ int s_row_start[kMaxGroups + 1];
@@ -55,7 +65,7 @@ void gmm_direct_kernel(const GmmArgs p) {
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave / WN, wn = wave % WN;
     const int E = p.E;
 
     build_work_list<kDM>(p, s_tile_start, s_row_start);
@@ -79,7 +89,7 @@ void gmm_direct_kernel(const GmmArgs p) {
 
     // ---- per-lane constants of the operand reads ----
     const int l31 = lane & 31, kgrp = lane >> 5;
-    const int fa_base = (wm * 128 + l31) * 64;
+    const int fa_base = (wm * TM + l31) * 64;
     const int f_sw = (l31 >> 2) & 3;
     const int g16 = lane >> 4, i16 = lane & 15;
 
@@ -89,7 +99,7 @@ void gmm_direct_kernel(const GmmArgs p) {
     // ---- state of the tile whose copies are being issued (set by open_tile) ----
     int e = 0, row0 = 0, rows_e = 0, n0 = 0;
     const char *a_base = nullptr, *b_exp = nullptr;
-    uint32_t a_off[4], b_off[4];
+    uint32_t a_off[CA], b_off[4];
 
     // tile column slot (0..255) -> column of b; slots past the end read the first column (never stored)
     auto b_col = [&](int slot) {
@@ -108,26 +118,29 @@ void gmm_direct_kernel(const GmmArgs p) {
         a_base = p.a + (long long)row0 * pitch;
         b_exp = p.b + (long long)e * p.K * p.N * 2;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < CA; ++i) {
             int r = (i * 4 + wave) * 16 + kc_row;
             if (r >= rows_e) r = rows_e - 1;                   // clamp: loaded, never stored
             a_off[i] = (uint32_t)r * pitch + kc_chunk * 16;
-            if constexpr (TRANS_B) b_off[i] = (uint32_t)b_col((i * 4 + wave) * 16 + kc_row) * pitch + kc_chunk * 16;
+        }
+        if constexpr (TRANS_B) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) b_off[i] = (uint32_t)b_col((i * 4 + wave) * 16 + kc_row) * pitch + kc_chunk * 16;
         }
         if constexpr (!TRANS_B) b_off[0] = (uint32_t)kn_k * (uint32_t)p.N * 2 + (uint32_t)b_col(kn_chunk * 8) * 2;
     };
 
-    // copy number c (0..7) of this wavefront for stage s: 0..3 are its A blocks, 4..7 its B blocks
+    // copy number c (0 .. kLoads-1) of this wavefront for stage s: first its CA blocks of A, then its 4 blocks of B
     auto issue_copy = [&](int s, int c) {
 #ifdef DMOE_DEBUG_HOOKS
         // timing experiments (wrong results): 1 = no copies after the prologue, 2 = no A copies, 3 = no B copies
-        if (s >= kStages && (p.dbg == 1 || (p.dbg == 2 && c < 4) || (p.dbg == 3 && c >= 4))) return;
+        if (s >= kStages && (p.dbg == 1 || (p.dbg == 2 && c < CA) || (p.dbg == 3 && c >= CA))) return;
 #endif
-        const uint32_t lA = smem_addr + (s & (kStages - 1)) * kStage + wave * 1024;
-        if (c < 4) {
+        const uint32_t lA = smem_addr + (s % kStages) * kStage + wave * 1024;
+        if (c < CA) {
             copy_g2lds_16(a_base + (long long)s * (kDK * 2) + a_off[c], lA + c * 4096);
         } else {
-            const int i = c - 4;
+            const int i = c - CA;
             const uint32_t lB = lA + kStageA + i * 4096;
             if constexpr (TRANS_B) copy_g2lds_16(b_exp + (long long)s * (kDK * 2) + b_off[i], lB);
             else copy_g2lds_16(b_exp + ((long long)s * kDK + i * 8) * p.N * 2 + b_off[0], lB);
@@ -142,10 +155,11 @@ void gmm_direct_kernel(const GmmArgs p) {
     };
 
     // B operand rows / columns of this wavefront: fragment j covers 32 tile columns
-    int fb_off[4];
+    int fb_off[FN];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const int slot0 = SWIGLU ? ((j < 2) ? wn * 64 + j * 32 : kDN / 2 + wn * 64 + (j - 2) * 32) : wn * 128 + j * 32;
+    for (int j = 0; j < FN; ++j) {
+        const int slot0 = SWIGLU ? ((j < FN / 2) ? wn * (TN / 2) + j * 32 : kDN / 2 + wn * (TN / 2) + (j - FN / 2) * 32)
+                                 : wn * TN + j * 32;
         if constexpr (TRANS_B) {
             fb_off[j] = (slot0 + l31) * 64;
         } else {
@@ -155,17 +169,18 @@ void gmm_direct_kernel(const GmmArgs p) {
         }
     }
 
-    bf16x8 fa[2][4], fb[2][4];
-    // operand read number r (0..7) of k-step ks of stage s into register set `slot`: 0..3 A, 4..7 B fragments
+    bf16x8 fa[2][FM], fb[2][FN];
+    // operand read number r (0 .. NR-1) of k-step ks of stage s into register set `slot`: first the FM A fragments,
+    // then the FN B fragments
     auto load_frag = [&](int s, int ks, int slot, int r) {
-        const char *tA = smem + (s & (kStages - 1)) * kStage;
+        const char *tA = smem + (s % kStages) * kStage;
         const char *tB = tA + kStageA;
         const int c0 = ((ks * 2 + kgrp) ^ f_sw) << 4;
-        if (r < 4) {
+        if (r < FM) {
             const u32x4 x = *(const u32x4 *)(tA + fa_base + r * 2048 + c0);
             __builtin_memcpy(&fa[slot][r], &x, 16);
         } else {
-            const int j = r - 4;
+            const int j = r - FM;
             if constexpr (TRANS_B) {
                 const u32x4 x = *(const u32x4 *)(tB + fb_off[j] + c0);
                 __builtin_memcpy(&fb[slot][j], &x, 16);
@@ -177,6 +192,16 @@ void gmm_direct_kernel(const GmmArgs p) {
                 __builtin_memcpy(&fb[slot][j], &v, 16);
             }
         }
+    };
+
+    // wait until at most n * kLoads of this wavefront's copies are outstanding (n known only at run time)
+    auto wait_ahead = [&](int n) {
+        if (n >= 5) DMOE_WAIT_VMCNT(5 * kLoads > 63 ? 63 : 5 * kLoads);
+        else if (n == 4) DMOE_WAIT_VMCNT(4 * kLoads > 63 ? 63 : 4 * kLoads);
+        else if (n == 3) DMOE_WAIT_VMCNT(3 * kLoads);
+        else if (n == 2) DMOE_WAIT_VMCNT(2 * kLoads);
+        else if (n == 1) DMOE_WAIT_VMCNT(kLoads);
+        else DMOE_WAIT_VMCNT(0);
     };
 
     // ---- first work item ----
@@ -197,75 +222,68 @@ void gmm_direct_kernel(const GmmArgs p) {
         // results of this tile go here after the next tile's copies have been issued
         const int cur_row0 = row0, cur_rows_e = rows_e, cur_n0 = n0;
         // row fragments of this wavefront that hold at least one valid row (a short last tile skips the rest)
-        int nfr = ((rows_e < kDM ? rows_e : kDM) - wm * 128 + 31) / 32;
-        nfr = nfr < 0 ? 0 : (nfr > 4 ? 4 : nfr);
+        int nfr = ((rows_e < kDM ? rows_e : kDM) - wm * TM + 31) / 32;
+        nfr = nfr < 0 ? 0 : (nfr > FM ? FM : nfr);
 
-        f32x16 acc[4][4];
+        f32x16 acc[FM][FN];
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < FM; ++i)
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
+            for (int j = 0; j < FN; ++j)
 #pragma unroll
                 for (int x = 0; x < 16; ++x) acc[i][j][x] = 0.f;
         auto mfma_one = [&](int slot, int t) {
-            const int i = t >> 2, j = t & 3;
+            const int i = t / FN, j = t % FN;
             if (i >= nfr) return;   // wave-uniform: a scalar branch around the MFMA
             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[slot][j], fa[slot][i], acc[i][j], 0, 0, 0);
         };
 
         // stage 0 of this tile has landed (its other prologue stages, and stores of the previous tile's
         // epilogue that were issued after them, may still be in flight: waiting for fewer is only stricter)
-        if (pre == 4) DMOE_WAIT_VMCNT(3 * kLoads);
-        else if (pre == 3) DMOE_WAIT_VMCNT(2 * kLoads);
-        else if (pre == 2) DMOE_WAIT_VMCNT(kLoads);
-        else DMOE_WAIT_VMCNT(0);
+        wait_ahead(pre - 1);
         __syncthreads();
 #pragma unroll
-        for (int r = 0; r < 8; ++r) load_frag(0, 0, 0, r);
+        for (int r = 0; r < NR; ++r) load_frag(0, 0, 0, r);
 
-        // One stage = 2 k-steps of 16 MFMAs.  A wavefront issues in order and an MFMA occupies the matrix
-        // pipe for 32 cycles, so the LDS reads and global -> LDS copies are slotted one per MFMA: they are
-        // issued in the shadow of the MFMA before them and the pipe never waits for the issue port.
-        //   k-step 0: MFMAs on register set 0; the 8 operand reads of k-step 1 go to set 1.
+        // One stage = 2 k-steps of NM MFMAs.  A wavefront issues in order and an MFMA occupies the matrix pipe
+        // for 32 cycles, so the LDS reads and global -> LDS copies are slotted one per MFMA: they are issued in
+        // the shadow of the MFMA before them and the pipe never waits for the issue port.
+        //   k-step 0: MFMAs on register set 0; the NR operand reads of k-step 1 go to set 1.
         //   hand-over: this wavefront's share of stage s+1 has landed (vmcnt), barrier (everybody's has, and
         //              every read of stage s is complete).
-        //   k-step 1: MFMAs on set 1; the 8 operand reads of stage s+1 go to set 0, then the 8 copies that
-        //              refill the LDS stage just drained with stage s+4.
-        // kAhead = stages after s+1 whose copies are already in flight when s+1 is opened.
-        auto run_stage = [&](int s, auto ahead_tag, auto next_tag, auto copy_tag) {
-            constexpr int kAhead = decltype(ahead_tag)::value;
-            constexpr bool kNext = decltype(next_tag)::value;
-            constexpr bool kCopy = decltype(copy_tag)::value;
+        //   k-step 1: MFMAs on set 1; the NR operand reads of stage s+1 go to set 0, then the copies that refill
+        //              the LDS stage just drained with stage s + kStages.
+        // kSteady: the copies of s+1 .. s+kStages-1 are in flight; otherwise `ahead` stages after s+1 are.
+        auto run_stage = [&](int s, auto steady_tag, int ahead, bool next) {
+            constexpr bool kSteady = decltype(steady_tag)::value;
 #pragma unroll
-            for (int t = 0; t < 16; ++t) {
+            for (int t = 0; t < NM; ++t) {
                 mfma_one(0, t);
-                if (t < 8) load_frag(s, 1, 1, t);
+                if (t < NR) load_frag(s, 1, 1, t);
                 __builtin_amdgcn_sched_barrier(0);
             }
-            if constexpr (kNext) {
-                DMOE_WAIT_VMCNT(kAhead * kLoads);
+            if (kSteady || next) {
+                if constexpr (kSteady) DMOE_WAIT_VMCNT((kStages - 2) * kLoads);
+                else wait_ahead(ahead);
                 __syncthreads();
                 __builtin_amdgcn_sched_barrier(0);
             }
 #pragma unroll
-            for (int t = 0; t < 16; ++t) {
-                mfma_one(1, t);
-                if constexpr (kNext) {
-                    if (t < 8) load_frag(s + 1, 0, 0, t);
-                    else if constexpr (kCopy) issue_copy(s + kStages, t - 8);
+            for (int t = 0; t < (NM > NR + kLoads ? NM : NR + kLoads); ++t) {
+                if (t < NM) mfma_one(1, t);
+                if (kSteady || next) {
+                    if (t < NR) load_frag(s + 1, 0, 0, t);
+                    else if (kSteady && t < NR + kLoads) issue_copy(s + kStages, t - NR);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
         };
-        typedef std::integral_constant<int, 2> two_t;
-        typedef std::integral_constant<int, 1> one_t;
-        typedef std::integral_constant<int, 0> zero_t;
         int s = 0;
-        for (; s + kStages < S; ++s) run_stage(s, two_t{}, std::true_type{}, std::true_type{});
-        if (s + 3 < S) { run_stage(s, two_t{}, std::true_type{}, std::false_type{}); ++s; }
-        if (s + 2 < S) { run_stage(s, one_t{}, std::true_type{}, std::false_type{}); ++s; }
-        if (s + 1 < S) { run_stage(s, zero_t{}, std::true_type{}, std::false_type{}); ++s; }
-        run_stage(s, zero_t{}, std::false_type{}, std::false_type{});
+        for (; s + kStages < S; ++s) run_stage(s, std::true_type{}, 0, true);
+        for (; s < S; ++s) {
+            const int left = S - 1 - s;                           // stages after this one
+            run_stage(s, std::false_type{}, left - 1 < kStages - 2 ? left - 1 : kStages - 2, left > 0);
+        }
 
         auto next_item = [&]() {
             // ---- next work item and its first copies ----
@@ -283,24 +301,24 @@ void gmm_direct_kernel(const GmmArgs p) {
             // The MFMAs take the B fragment as their first operand, so an accumulator holds the tile transposed:
             // lane l owns output row l % 32 of its fragment and, in element x, column (x/4)*8 + (l/32)*4 + x%4.
             // Four consecutive columns per lane -> one 8-byte store; a row is valid or not per lane.
-            constexpr int FNO = SWIGLU ? 2 : 4;
-    #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int r = wm * 128 + i * 32 + l31;
+            constexpr int FNO = SWIGLU ? FN / 2 : FN;
+#pragma unroll
+            for (int i = 0; i < FM; ++i) {
+                const int r = wm * TM + i * 32 + l31;
                 if (r >= cur_rows_e) continue;
-                const int col_lane = cur_n0 + (SWIGLU ? wn * 64 : wn * 128) + kgrp * 4;
+                const int col_lane = cur_n0 + (SWIGLU ? wn * (TN / 2) : wn * TN) + kgrp * 4;
                 uint16_t *crow = (uint16_t *)p.c + (long long)(cur_row0 + r) * p.ldc + col_lane;
-    #pragma unroll
+#pragma unroll
                 for (int j = 0; j < FNO; ++j) {
-    #pragma unroll
+#pragma unroll
                     for (int g = 0; g < 4; ++g) {
                         if (col_lane + j * 32 + g * 8 >= n_out) continue;   // n_out % 8 == 0: four columns at once
                         float v[4];
-    #pragma unroll
+#pragma unroll
                         for (int x = 0; x < 4; ++x) {
                             if (SWIGLU) {
                                 const float gate = acc[i][j][g * 4 + x];
-                                v[x] = silu_mul(gate, acc[i][j + 2][g * 4 + x]);
+                                v[x] = silu_mul(gate, acc[i][j + FN / 2][g * 4 + x]);
                             } else {
                                 v[x] = acc[i][j][g * 4 + x];
                             }
@@ -310,7 +328,7 @@ void gmm_direct_kernel(const GmmArgs p) {
                         packed.y = pack_bf16x2(v[2], v[3]);
 #ifdef DMOE_DEBUG_HOOKS
                         if (p.dbg == 7) {   // timing experiment: same bytes, fully coalesced addresses (wrong results)
-                            uint2 *lin = (uint2 *)((uint16_t *)p.c + (long long)cur_row0 * p.ldc) + ((wave * 64 + (i * 16 + j * 4 + g)) * 64 + lane);
+                            uint2 *lin = (uint2 *)((uint16_t *)p.c + (long long)cur_row0 * p.ldc) + ((wave * 64 + (i * FN * 4 + j * 4 + g)) * 64 + lane);
                             *lin = packed;
                             continue;
                         }
@@ -335,11 +353,12 @@ void gmm_direct_kernel(const GmmArgs p) {
     sched_finish(p.sched_slot);
 }
 
-template <bool TRANS_B, bool SWIGLU>
+template <int kDM, int WM, bool TRANS_B, bool SWIGLU>
 static int launch_direct_one(const GmmArgs &args, hipStream_t stream) {
     constexpr int BNO = SWIGLU ? kDN / 2 : kDN;
-    const size_t lds = (size_t)kStages * kStage;
-    auto kern = gmm_direct_kernel<TRANS_B, SWIGLU>;
+    constexpr int kStages = kDM == 256 ? 4 : (kDM == 128 ? 5 : 6);
+    const size_t lds = (size_t)kStages * (kDM * kDK * 2 + kStageB);
+    auto kern = gmm_direct_kernel<kDM, WM, TRANS_B, SWIGLU>;
     static bool configured = false;
     if (!configured) {
         DMOE_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
@@ -359,10 +378,18 @@ static int launch_direct_one(const GmmArgs &args, hipStream_t stream) {
     return DMOE_OK;
 }
 
+template <int kDM, int WM>
+static int launch_direct_tile(const GmmArgs &args, bool trans_b, bool swiglu, hipStream_t stream) {
+    if (trans_b) return swiglu ? launch_direct_one<kDM, WM, true, true>(args, stream) : launch_direct_one<kDM, WM, true, false>(args, stream);
+    return swiglu ? launch_direct_one<kDM, WM, false, true>(args, stream) : launch_direct_one<kDM, WM, false, false>(args, stream);
+}
+
 // Preconditions (checked by the caller): bf16, K % 32 == 0, N % 8 == 0, K * N * 2 < 2^32.
-int launch_direct_bf16(const GmmArgs &args, bool trans_b, bool swiglu, hipStream_t stream) {
-    if (trans_b) return swiglu ? launch_direct_one<true, true>(args, stream) : launch_direct_one<true, false>(args, stream);
-    return swiglu ? launch_direct_one<false, true>(args, stream) : launch_direct_one<false, false>(args, stream);
+// tile_rows: 256, 128 or 64.
+int launch_direct_bf16(const GmmArgs &args, int tile_rows, bool trans_b, bool swiglu, hipStream_t stream) {
+    if (tile_rows == 64) return launch_direct_tile<64, 1>(args, trans_b, swiglu, stream);
+    if (tile_rows == 128) return launch_direct_tile<128, 2>(args, trans_b, swiglu, stream);
+    return launch_direct_tile<256, 2>(args, trans_b, swiglu, stream);
 }
 
 }  // namespace dmoe

@@ -113,11 +113,7 @@ void gmm_kernel(const GmmArgs p) {
         // ---- staging offsets (bytes from wave-uniform bases) ----
         const char *a_base = p.a + (long long)row0 * a_pitch;
         const char *b_exp = p.b + (long long)e * p.K * p.N * ES;
-#ifdef DMOE_DBG_SAME_B
-        const int n0_b = 0;       // timing experiment: every n-tile reads the first weight tile (wrong results)
-#else
         const int n0_b = n0;
-#endif
         // first column of the tile; the swiglu form reads a second run of columns (the up half)
         const char *b_base0, *b_base1;
         if constexpr (TRANS_B) {
@@ -181,9 +177,6 @@ void gmm_kernel(const GmmArgs p) {
         };
         const int KT_full = (p.K * ES) / kRowBytes;            // tiles that lie inside K entirely
         auto load_tile = [&](int kt) {
-#ifdef DMOE_DBG_NO_GLOAD
-            if (kt > 1) return;   // timing experiment: no global traffic after the prologue (wrong results)
-#endif
             if (kt < KT_full) load_global(kt, std::false_type{});
             else load_global(kt, std::true_type{});
         };
@@ -450,6 +443,11 @@ static int launch_by_rows(const GmmArgs &args, hipStream_t stream) {
         // global -> LDS direct path: whole stages of 32 k, 32-bit offsets inside one expert's weights
         if (args.K % 32 == 0 && (long long)args.K * args.N * 2 < (1ll << 32))
             return launch_direct_bf16(args, tile_rows, TRANS_B, SWIGLU, stream);
+    } else {
+        // measured on the 8x22b shapes: with 256-row tiles the register-staged 8-wave kernel is ahead for the fused
+        // gate-up projection, the direct kernel (128-row tiles at most) for the plain product
+        if (args.K % 64 == 0 && (long long)args.K * args.N < (1ll << 32) && !(SWIGLU && tile_rows == 256))
+            return launch_direct_fp8(args, tile_rows, SWIGLU, stream);
     }
     if (tile_rows == 64) return launch_one<64, 256, 1, 4, TRANS_B, SWIGLU, FP8>(args, stream);
     if (tile_rows == 128) return launch_one<128, 256, 1, 4, TRANS_B, SWIGLU, FP8>(args, stream);

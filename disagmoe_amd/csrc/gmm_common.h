@@ -168,5 +168,6 @@ __device__ __forceinline__ TileCoord decode_tile(long long q, int G, long long t
 
 int next_sched_slot();
 int launch_direct_bf16(const GmmArgs &args, int tile_rows, bool trans_b, bool swiglu, hipStream_t stream);
+int launch_direct_fp8(const GmmArgs &args, int tile_rows, bool swiglu, hipStream_t stream);
 
 }  // namespace dmoe

@@ -1,4 +1,4 @@
-// bf16 grouped GEMM on the CDNA4 data path: tiles of 256, 128 or 64 rows by 256 columns.
+// bf16 (and fp8 e4m3) grouped GEMM on the CDNA4 data path: tiles of 256, 128 or 64 rows by 256 columns.
 //
 //   * A and B tiles go global -> LDS directly (global_load_lds_dwordx4: each lane
 //     fetches 16 bytes, the wavefront fills 1 KiB of LDS), no staging registers,
@@ -41,9 +41,13 @@ constexpr int kStageB = kDN * kDK * 2;     // 16 KiB of B per stage
 // s_waitcnt with only vmcnt set (gfx9 encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14)
 #define DMOE_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (7 << 4) | (15 << 8) | (((n) >> 4) << 14))
 
-template <int kDM, int WM, bool TRANS_B, bool SWIGLU>
+// FP8: operands are e4m3 bytes, K-contiguous on both sides (TRANS_B), a stage holds 64 k = one
+// v_mfma_f32_32x32x64_f8f6f4 k-step, and per-row / per-column scales are applied in the epilogue.
+template <int kDM, int WM, bool TRANS_B, bool SWIGLU, bool FP8>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
 void gmm_direct_kernel(const GmmArgs p) {
+    constexpr int kStageK = FP8 ? 64 : kDK;               // k per stage: 64 bytes per row either way
+    static_assert(!FP8 || TRANS_B, "fp8 operands are K-contiguous");
     constexpr int WN = 4 / WM;                           // wavefronts along N
     constexpr int TM = kDM / WM, TN = kDN / WN;          // wave tile
     constexpr int FM = TM / 32, FN = TN / 32;            // 32x32 accumulators per wavefront
@@ -64,7 +68,7 @@ void gmm_direct_kernel(const GmmArgs p) {
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // kept in a scalar register: what derives from it stays wave-uniform
     const int wm = wave / WN, wn = wave % WN;
     const int E = p.E;
 
@@ -74,9 +78,9 @@ void gmm_direct_kernel(const GmmArgs p) {
     const int n_out = SWIGLU ? p.N / 2 : p.N;
     const int n_tiles = (n_out + BNO - 1) / BNO;
     const long long total = (long long)s_tile_start[E] * n_tiles;
-    const int S = p.K / kDK;                       // stages (K % 32 == 0)
+    const int S = p.K / kStageK;                   // stages (whole stages only)
     const int G = gridDim.x;
-    const uint32_t pitch = (uint32_t)p.K * 2;      // bytes per row of a (and of b when K-contiguous)
+    const uint32_t pitch = (uint32_t)p.K * (FP8 ? 1 : 2);   // bytes per row of a (and of b when K-contiguous)
     const uint32_t smem_addr = lds_addr(smem);
 
     // ---- per-lane constants of the global -> LDS copies ----
@@ -116,7 +120,7 @@ void gmm_direct_kernel(const GmmArgs p) {
         const TileCoord tc = decode_tile<kDM>(q, G, total, n_tiles, E, s_tile_start, s_row_start);
         e = tc.e; row0 = tc.row0; rows_e = tc.rows_e; n0 = tc.nt * BNO;
         a_base = p.a + (long long)row0 * pitch;
-        b_exp = p.b + (long long)e * p.K * p.N * 2;
+        b_exp = p.b + (long long)e * p.K * p.N * (FP8 ? 1 : 2);
 #pragma unroll
         for (int i = 0; i < CA; ++i) {
             int r = (i * 4 + wave) * 16 + kc_row;
@@ -138,11 +142,11 @@ void gmm_direct_kernel(const GmmArgs p) {
 #endif
         const uint32_t lA = smem_addr + (s % kStages) * kStage + wave * 1024;
         if (c < CA) {
-            copy_g2lds_16(a_base + (long long)s * (kDK * 2) + a_off[c], lA + c * 4096);
+            copy_g2lds_16(a_base + (long long)s * 64 + a_off[c], lA + c * 4096);
         } else {
             const int i = c - CA;
             const uint32_t lB = lA + kStageA + i * 4096;
-            if constexpr (TRANS_B) copy_g2lds_16(b_exp + (long long)s * (kDK * 2) + b_off[i], lB);
+            if constexpr (TRANS_B) copy_g2lds_16(b_exp + (long long)s * 64 + b_off[i], lB);
             else copy_g2lds_16(b_exp + ((long long)s * kDK + i * 8) * p.N * 2 + b_off[0], lB);
         }
     };
@@ -169,14 +173,24 @@ void gmm_direct_kernel(const GmmArgs p) {
         }
     }
 
-    bf16x8 fa[2][FM], fb[2][FN];
+    typedef typename std::conditional<FP8, i32x8, bf16x8>::type frag_t;
+    frag_t fa[FP8 ? 1 : 2][FM], fb[2][FN];
     // operand read number r (0 .. NR-1) of k-step ks of stage s into register set `slot`: first the FM A fragments,
     // then the FN B fragments
     auto load_frag = [&](int s, int ks, int slot, int r) {
         const char *tA = smem + (s % kStages) * kStage;
         const char *tB = tA + kStageA;
         const int c0 = ((ks * 2 + kgrp) ^ f_sw) << 4;
-        if (r < FM) {
+        if constexpr (FP8) {
+            // a lane holds 32 consecutive k of its row: chunks 2*kgrp and 2*kgrp + 1 of the 64-byte row
+            const int d0 = ((kgrp * 2) ^ f_sw) << 4, d1 = ((kgrp * 2 + 1) ^ f_sw) << 4;
+            const char *src = r < FM ? tA + fa_base + r * 2048 : tB + fb_off[r - FM];
+            const u32x4 x0 = *(const u32x4 *)(src + d0);
+            const u32x4 x1 = *(const u32x4 *)(src + d1);
+            const i32x8 v = {(int)x0[0], (int)x0[1], (int)x0[2], (int)x0[3], (int)x1[0], (int)x1[1], (int)x1[2], (int)x1[3]};
+            if (r < FM) __builtin_memcpy(&fa[slot][r], &v, 32);
+            else __builtin_memcpy(&fb[slot][r - FM], &v, 32);
+        } else if (r < FM) {
             const u32x4 x = *(const u32x4 *)(tA + fa_base + r * 2048 + c0);
             __builtin_memcpy(&fa[slot][r], &x, 16);
         } else {
@@ -220,7 +234,7 @@ void gmm_direct_kernel(const GmmArgs p) {
 
     while (q < total) {
         // results of this tile go here after the next tile's copies have been issued
-        const int cur_row0 = row0, cur_rows_e = rows_e, cur_n0 = n0;
+        const int cur_row0 = row0, cur_rows_e = rows_e, cur_n0 = n0, cur_e = e;
         // row fragments of this wavefront that hold at least one valid row (a short last tile skips the rest)
         int nfr = ((rows_e < kDM ? rows_e : kDM) - wm * TM + 31) / 32;
         nfr = nfr < 0 ? 0 : (nfr > FM ? FM : nfr);
@@ -235,7 +249,14 @@ void gmm_direct_kernel(const GmmArgs p) {
         auto mfma_one = [&](int slot, int t) {
             const int i = t / FN, j = t % FN;
             if (i >= nfr) return;   // wave-uniform: a scalar branch around the MFMA
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[slot][j], fa[slot][i], acc[i][j], 0, 0, 0);
+            if constexpr (!FP8)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[slot][j], fa[slot][i], acc[i][j], 0, 0, 0);
+        };
+        auto mfma_one_fp8 = [&](int bslot, int t) {
+            const int i = t / FN, j = t % FN;
+            if (i >= nfr) return;
+            if constexpr (FP8)
+                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[bslot][j], fa[0][i], acc[i][j], 0, 0, 0, 0, 0, 0);
         };
 
         // stage 0 of this tile has landed (its other prologue stages, and stores of the previous tile's
@@ -254,13 +275,18 @@ void gmm_direct_kernel(const GmmArgs p) {
         //   k-step 1: MFMAs on set 1; the NR operand reads of stage s+1 go to set 0, then the copies that refill
         //              the LDS stage just drained with stage s + kStages.
         // kSteady: the copies of s+1 .. s+kStages-1 are in flight; otherwise `ahead` stages after s+1 are.
-        auto run_stage = [&](int s, auto steady_tag, int ahead, bool next) {
+        // FP8: a stage is a single k-step, so the hand-over comes first and the register sets alternate by stage:
+        // MFMAs of stage s run on set s % 2 while stage s+1 is read into the other set.
+        auto run_stage = [&](int s, auto steady_tag, int ahead, bool next, auto odd_tag) {
             constexpr bool kSteady = decltype(steady_tag)::value;
+            constexpr int kCur = FP8 ? (decltype(odd_tag)::value ? 1 : 0) : 1;   // set used by the MFMAs after the hand-over
+            if constexpr (!FP8) {
 #pragma unroll
-            for (int t = 0; t < NM; ++t) {
-                mfma_one(0, t);
-                if (t < NR) load_frag(s, 1, 1, t);
-                __builtin_amdgcn_sched_barrier(0);
+                for (int t = 0; t < NM; ++t) {
+                    mfma_one(0, t);
+                    if (t < NR) load_frag(s, 1, 1, t);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
             if (kSteady || next) {
                 if constexpr (kSteady) DMOE_WAIT_VMCNT((kStages - 2) * kLoads);
@@ -268,21 +294,47 @@ void gmm_direct_kernel(const GmmArgs p) {
                 __syncthreads();
                 __builtin_amdgcn_sched_barrier(0);
             }
+            if constexpr (FP8) {
+                // 8 registers per operand: A fragments live in one register set and are re-read for stage s+1
+                // right behind their last MFMA of this stage; B fragments alternate between two sets.
 #pragma unroll
-            for (int t = 0; t < (NM > NR + kLoads ? NM : NR + kLoads); ++t) {
-                if (t < NM) mfma_one(1, t);
-                if (kSteady || next) {
-                    if (t < NR) load_frag(s + 1, 0, 0, t);
-                    else if (kSteady && t < NR + kLoads) issue_copy(s + kStages, t - NR);
+                for (int t = 0; t < (NM > FN + kLoads ? NM : FN + kLoads); ++t) {
+                    if (t < NM) mfma_one_fp8(kCur, t);
+                    if (kSteady || next) {
+                        if (t < FN) load_frag(s + 1, 0, kCur ^ 1, FM + t);
+                        else if (kSteady && t < FN + kLoads) issue_copy(s + kStages, t - FN);
+                        if (t < NM && (t % FN) == FN - 1) load_frag(s + 1, 0, 0, t / FN);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
                 }
-                __builtin_amdgcn_sched_barrier(0);
+            } else {
+#pragma unroll
+                for (int t = 0; t < (NM > NR + kLoads ? NM : NR + kLoads); ++t) {
+                    if (t < NM) mfma_one(kCur, t);
+                    if (kSteady || next) {
+                        if (t < NR) load_frag(s + 1, 0, kCur ^ 1, t);
+                        else if (kSteady && t < NR + kLoads) issue_copy(s + kStages, t - NR);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
         };
+        auto step = [&](int s, auto steady_tag, int ahead, bool next) {
+            if (FP8 && (s & 1)) run_stage(s, steady_tag, ahead, next, std::true_type{});
+            else run_stage(s, steady_tag, ahead, next, std::false_type{});
+        };
         int s = 0;
-        for (; s + kStages < S; ++s) run_stage(s, std::true_type{}, 0, true);
+        if constexpr (FP8) {
+            // even and odd stages as one straight-line loop body: the accumulators stay where they are
+            for (; s + 1 + kStages < S; s += 2) {
+                run_stage(s, std::true_type{}, 0, true, std::false_type{});
+                run_stage(s + 1, std::true_type{}, 0, true, std::true_type{});
+            }
+        }
+        for (; s + kStages < S; ++s) step(s, std::true_type{}, 0, true);
         for (; s < S; ++s) {
             const int left = S - 1 - s;                           // stages after this one
-            run_stage(s, std::false_type{}, left - 1 < kStages - 2 ? left - 1 : kStages - 2, left > 0);
+            step(s, std::false_type{}, left - 1 < kStages - 2 ? left - 1 : kStages - 2, left > 0);
         }
 
         auto next_item = [&]() {
@@ -308,19 +360,31 @@ void gmm_direct_kernel(const GmmArgs p) {
                 if (r >= cur_rows_e) continue;
                 const int col_lane = cur_n0 + (SWIGLU ? wn * (TN / 2) : wn * TN) + kgrp * 4;
                 uint16_t *crow = (uint16_t *)p.c + (long long)(cur_row0 + r) * p.ldc + col_lane;
+                float sa = 1.f;
+                if constexpr (FP8) sa = p.a_scale[cur_row0 + r];
 #pragma unroll
                 for (int j = 0; j < FNO; ++j) {
 #pragma unroll
                     for (int g = 0; g < 4; ++g) {
-                        if (col_lane + j * 32 + g * 8 >= n_out) continue;   // n_out % 8 == 0: four columns at once
+                        const int col = col_lane + j * 32 + g * 8;
+                        if (col >= n_out) continue;   // n_out % 8 == 0: four columns at once
+                        float sb0[4] = {1.f, 1.f, 1.f, 1.f}, sb1[4] = {1.f, 1.f, 1.f, 1.f};
+                        if constexpr (FP8) {
+                            const float4 t0 = *(const float4 *)(p.b_scale + (long long)cur_e * p.N + col);
+                            sb0[0] = t0.x; sb0[1] = t0.y; sb0[2] = t0.z; sb0[3] = t0.w;
+                            if (SWIGLU) {
+                                const float4 t1 = *(const float4 *)(p.b_scale + (long long)cur_e * p.N + n_out + col);
+                                sb1[0] = t1.x; sb1[1] = t1.y; sb1[2] = t1.z; sb1[3] = t1.w;
+                            }
+                        }
                         float v[4];
 #pragma unroll
                         for (int x = 0; x < 4; ++x) {
                             if (SWIGLU) {
-                                const float gate = acc[i][j][g * 4 + x];
-                                v[x] = silu_mul(gate, acc[i][j + FN / 2][g * 4 + x]);
+                                const float gate = acc[i][j][g * 4 + x] * (sa * sb0[x]);
+                                v[x] = silu_mul(gate, acc[i][j + FN / 2][g * 4 + x] * (sa * sb1[x]));
                             } else {
-                                v[x] = acc[i][j][g * 4 + x];
+                                v[x] = acc[i][j][g * 4 + x] * (sa * sb0[x]);
                             }
                         }
                         uint2 packed;
@@ -353,12 +417,12 @@ void gmm_direct_kernel(const GmmArgs p) {
     sched_finish(p.sched_slot);
 }
 
-template <int kDM, int WM, bool TRANS_B, bool SWIGLU>
+template <int kDM, int WM, bool TRANS_B, bool SWIGLU, bool FP8>
 static int launch_direct_one(const GmmArgs &args, hipStream_t stream) {
     constexpr int BNO = SWIGLU ? kDN / 2 : kDN;
     constexpr int kStages = kDM == 256 ? 4 : (kDM == 128 ? 5 : 6);
     const size_t lds = (size_t)kStages * (kDM * kDK * 2 + kStageB);
-    auto kern = gmm_direct_kernel<kDM, WM, TRANS_B, SWIGLU>;
+    auto kern = gmm_direct_kernel<kDM, WM, TRANS_B, SWIGLU, FP8>;
     static bool configured = false;
     if (!configured) {
         DMOE_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
@@ -380,8 +444,8 @@ static int launch_direct_one(const GmmArgs &args, hipStream_t stream) {
 
 template <int kDM, int WM>
 static int launch_direct_tile(const GmmArgs &args, bool trans_b, bool swiglu, hipStream_t stream) {
-    if (trans_b) return swiglu ? launch_direct_one<kDM, WM, true, true>(args, stream) : launch_direct_one<kDM, WM, true, false>(args, stream);
-    return swiglu ? launch_direct_one<kDM, WM, false, true>(args, stream) : launch_direct_one<kDM, WM, false, false>(args, stream);
+    if (trans_b) return swiglu ? launch_direct_one<kDM, WM, true, true, false>(args, stream) : launch_direct_one<kDM, WM, true, false, false>(args, stream);
+    return swiglu ? launch_direct_one<kDM, WM, false, true, false>(args, stream) : launch_direct_one<kDM, WM, false, false, false>(args, stream);
 }
 
 // Preconditions (checked by the caller): bf16, K % 32 == 0, N % 8 == 0, K * N * 2 < 2^32.
@@ -390,6 +454,13 @@ int launch_direct_bf16(const GmmArgs &args, int tile_rows, bool trans_b, bool sw
     if (tile_rows == 64) return launch_direct_tile<64, 1>(args, trans_b, swiglu, stream);
     if (tile_rows == 128) return launch_direct_tile<128, 2>(args, trans_b, swiglu, stream);
     return launch_direct_tile<256, 2>(args, trans_b, swiglu, stream);
+}
+
+// Preconditions: e4m3 operands, K-contiguous on both sides, K % 64 == 0, N % 8 == 0, K * N < 2^32.
+int launch_direct_fp8(const GmmArgs &args, int tile_rows, bool swiglu, hipStream_t stream) {
+    if (tile_rows == 64) return swiglu ? launch_direct_one<64, 1, true, true, true>(args, stream) : launch_direct_one<64, 1, true, false, true>(args, stream);
+    // 256-row tiles would need 256 accumulator + 96 operand registers per lane plus addressing: they are cut in two
+    return swiglu ? launch_direct_one<128, 2, true, true, true>(args, stream) : launch_direct_one<128, 2, true, false, true>(args, stream);
 }
 
 }  // namespace dmoe

@@ -11,7 +11,7 @@ LIB_PATH = os.environ.get("DMOE_HIP_LIB") or os.path.join(_HERE, "libdmoe_hip.so
 
 # dmoe.h constants
 OK = 0
-BF16, FP16, FP8_E4M3 = 0, 1, 2
+BF16, FP16, FP8_E4M3, FP32 = 0, 1, 2, 3
 I32, I64 = 4, 8
 ORDER_REFERENCE, ORDER_STABLE = 0, 1
 COMBINE_FP32, COMBINE_REFERENCE = 0, 1
@@ -24,6 +24,7 @@ SIGNATURES = {
     "dmoe_route_scratch_bytes": (c_int, [c_int64, c_int, POINTER(c_size_t)]),
     "dmoe_route": (c_int, [c_void_p, c_int, c_int64, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p,
                            c_void_p, c_size_t, c_void_p]),
+    "dmoe_topk_softmax": (c_int, [c_void_p, c_int, c_int64, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p]),
     "dmoe_permute": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int, c_void_p,
                              c_void_p]),
     "dmoe_gather_rows": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int, c_void_p]),

@@ -39,6 +39,7 @@ extern "C" {
 #define DMOE_BF16 0
 #define DMOE_FP16 1
 #define DMOE_FP8_E4M3 2 /* OCP e4m3fn, max 448 */
+#define DMOE_FP32 3     /* router logits only */
 
 /* integer types of ids / mappings: the size in bytes */
 #define DMOE_I32 4
@@ -76,6 +77,21 @@ int dmoe_route_scratch_bytes(int64_t R, int E, size_t *bytes);
 int dmoe_route(const void *ids, int ids_type, int64_t R, int E, int order,
                void *mappings, int map_type, int64_t *batch_sizes, int64_t *offsets,
                void *scratch, size_t scratch_bytes, void *stream);
+
+/* ---- routing producer ---------------------------------------------------
+ * dmoe_topk_softmax replaces vllm's fused_topk(hidden_states, gating_output,
+ * topk, renormalize) as the attention side calls it
+ * (disagmoe/models/attention.py:228-231): softmax over the E router logits of
+ * a token in fp32, the k largest probabilities and their expert ids, and with
+ * renormalize != 0 the k weights divided by their sum.  Ties go to the lower
+ * expert id.  The ids feed dmoe_route without visiting the host.
+ *
+ *   logits   [n, E]  DMOE_FP32, DMOE_BF16 or DMOE_FP16, E <= 1024
+ *   weights  [n, k]  fp32, descending
+ *   ids      [n, k]  DMOE_I32 (what fused_topk returns) or DMOE_I64, k <= 32
+ */
+int dmoe_topk_softmax(const void *logits, int logits_dtype, int64_t n, int E, int k, int renormalize,
+                      float *weights, void *ids, int ids_type, void *stream);
 
 /* ---- row movement -------------------------------------------------------
  * dmoe_permute replaces permute_tokens_cuda(tokens, mappings, stream)

@@ -21,6 +21,9 @@ formula) is listed below; the checks live in ``tests/test_oracle_*.py``.
   routing.expert_batch_sizes           ``numpy.bincount`` + index select.
   routing.sort_by_prefill_order        the reference's own known answer
       (tests/engine/test_exp_engine.py:29-40) in tests/golden/prefill_kat.json.
+  routing.fused_topk                   closed forms: logits ``ln(1..E)`` give
+      probabilities ``i / sum``; renormalised weights equal the softmax over the
+      kept logits alone (float64); brute-force selection on small inputs; ties.
   rows.permute_tokens / gather_rows    the reference test's row loop
       (tests/ops/test_memory.py:27-31) and ``torch.index_select``.
   ffn.gmm                               E=1 equals ``torch.matmul``; float64

@@ -135,3 +135,30 @@ def apply_row_mapping(values: Sequence, mapping: Sequence[int]) -> list:
     for i, m in enumerate(mapping):
         out[m] = values[i]
     return out
+
+
+def fused_topk(gating_output, topk: int, renormalize: bool = True):
+    """Routing producer ``fused_topk(hidden_states, gating_output, topk,
+    renormalize)`` of vllm 0.6.2 (requirements.txt:5; not present in this
+    checkout), as called at disagmoe/models/attention.py:228-231.  Its published
+    definition: ``w = softmax(gating_output.float(), dim=-1)``; the ``topk``
+    largest ``w`` per token with their expert ids; with ``renormalize`` divide
+    the kept weights by their sum.  Ties go to the lower expert id (vllm's
+    ``topk_softmax`` kernel scans experts upwards and replaces only on a strictly
+    larger value).  The order is taken on the logits, which is the order of the
+    probabilities wherever their fp32 rounding keeps distinct logits apart.
+    Returns ``(weights [n, topk] float32, ids [n, topk] int32)``."""
+    x = gating_output
+    if hasattr(x, "detach"):
+        x = x.detach().cpu().float().numpy()
+    x = np.asarray(x, dtype=np.float32)
+    n, E = x.shape
+    assert 1 <= topk <= E
+    order = np.argsort(-x.astype(np.float64), axis=1, kind="stable")[:, :topk]   # stable: lower id first among equals
+    m = x.max(axis=1, keepdims=True)
+    p = np.exp((x - m).astype(np.float32)).astype(np.float32)
+    p = p / p.sum(axis=1, keepdims=True, dtype=np.float32)
+    w = np.take_along_axis(p, order, axis=1).astype(np.float32)
+    if renormalize:
+        w = w / w.sum(axis=1, keepdims=True, dtype=np.float32)
+    return w.astype(np.float32), order.astype(np.int32)

@@ -126,10 +126,20 @@ void gmm_direct_kernel(const GmmArgs p) {
             int r = (i * 4 + wave) * 16 + kc_row;
             if (r >= rows_e) r = rows_e - 1;                   // clamp: loaded, never stored
             a_off[i] = (uint32_t)r * pitch + kc_chunk * 16;
+#ifdef DMOE_DEBUG_HOOKS
+            // timing experiment 8 (wrong results): whole 128-byte lines, 8 rows per copy, the other 8 rows on odd stages
+            if (p.dbg == 8) a_off[i] = (uint32_t)((i * 4 + wave) * 16 + (lane >> 3)) * pitch + (lane & 7) * 16;
+#endif
         }
         if constexpr (TRANS_B) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) b_off[i] = (uint32_t)b_col((i * 4 + wave) * 16 + kc_row) * pitch + kc_chunk * 16;
+#ifdef DMOE_DEBUG_HOOKS
+            if (p.dbg == 8) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) b_off[i] = (uint32_t)b_col((i * 4 + wave) * 16 + (lane >> 3)) * pitch + (lane & 7) * 16;
+            }
+#endif
         }
         if constexpr (!TRANS_B) b_off[0] = (uint32_t)kn_k * (uint32_t)p.N * 2 + (uint32_t)b_col(kn_chunk * 8) * 2;
     };
@@ -141,6 +151,21 @@ void gmm_direct_kernel(const GmmArgs p) {
         if (s >= kStages && (p.dbg == 1 || (p.dbg == 2 && c < CA) || (p.dbg == 3 && c >= CA))) return;
 #endif
         const uint32_t lA = smem_addr + (s % kStages) * kStage + wave * 1024;
+#ifdef DMOE_DEBUG_HOOKS
+        if (p.dbg == 9) {   // timing experiment (wrong results): every stage fetches the bytes of stage 0 again
+            const uint32_t lA9 = smem_addr + (s % kStages) * kStage + wave * 1024;
+            if (c < CA) copy_g2lds_16(a_base + a_off[c], lA9 + c * 4096);
+            else if constexpr (TRANS_B) copy_g2lds_16(b_exp + b_off[c - CA], lA9 + kStageA + (c - CA) * 4096);
+            else copy_g2lds_16(b_exp + ((long long)(c - CA) * 8) * p.N * 2 + b_off[0], lA9 + kStageA + (c - CA) * 4096);
+            return;
+        }
+        if (p.dbg == 8 && TRANS_B) {
+            const long long line = (long long)(s >> 1) * 128 + (long long)(s & 1) * 8 * pitch;
+            if (c < CA) copy_g2lds_16(a_base + line + a_off[c], lA + c * 4096);
+            else copy_g2lds_16(b_exp + line + b_off[c - CA], lA + kStageA + (c - CA) * 4096);
+            return;
+        }
+#endif
         if (c < CA) {
             copy_g2lds_16(a_base + (long long)s * 64 + a_off[c], lA + c * 4096);
         } else {
@@ -237,8 +262,13 @@ void gmm_direct_kernel(const GmmArgs p) {
         const int cur_row0 = row0, cur_rows_e = rows_e, cur_n0 = n0, cur_e = e;
         // row fragments of this wavefront that hold at least one valid row (a short last tile skips the rest)
         int nfr = ((rows_e < kDM ? rows_e : kDM) - wm * TM + 31) / 32;
-        nfr = nfr < 0 ? 0 : (nfr > FM ? FM : nfr);
+        nfr = __builtin_amdgcn_readfirstlane(nfr < 0 ? 0 : (nfr > FM ? FM : nfr));
 
+        // The tile from its first MFMA to its last store, in two builds: without any branch around the MFMAs (every
+        // row fragment of this wavefront holds rows: all but the last tile of an expert) and with one per MFMA.
+        // Wavefronts of one workgroup may take different builds; both execute the same copies and barriers.
+        auto run_tile = [&](auto guard_tag) {
+        constexpr bool kGuard = decltype(guard_tag)::value;
         f32x16 acc[FM][FN];
 #pragma unroll
         for (int i = 0; i < FM; ++i)
@@ -248,13 +278,13 @@ void gmm_direct_kernel(const GmmArgs p) {
                 for (int x = 0; x < 16; ++x) acc[i][j][x] = 0.f;
         auto mfma_one = [&](int slot, int t) {
             const int i = t / FN, j = t % FN;
-            if (i >= nfr) return;   // wave-uniform: a scalar branch around the MFMA
+            if (kGuard && i >= nfr) return;   // wave-uniform: a scalar branch around the MFMA
             if constexpr (!FP8)
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[slot][j], fa[slot][i], acc[i][j], 0, 0, 0);
         };
         auto mfma_one_fp8 = [&](int bslot, int t) {
             const int i = t / FN, j = t % FN;
-            if (i >= nfr) return;
+            if (kGuard && i >= nfr) return;
             if constexpr (FP8)
                 acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[bslot][j], fa[0][i], acc[i][j], 0, 0, 0, 0, 0, 0);
         };
@@ -272,19 +302,28 @@ void gmm_direct_kernel(const GmmArgs p) {
         //   k-step 0: MFMAs on register set 0; the NR operand reads of k-step 1 go to set 1.
         //   hand-over: this wavefront's share of stage s+1 has landed (vmcnt), barrier (everybody's has, and
         //              every read of stage s is complete).
-        //   k-step 1: MFMAs on set 1; the NR operand reads of stage s+1 go to set 0, then the copies that refill
-        //              the LDS stage just drained with stage s + kStages.
+        //   k-step 1: MFMAs on set 1; the NR operand reads of stage s+1 go to set 0; the copies that refill the LDS
+        //              stage just drained with stage s + kStages are spread over this k-step and the next one.
         // kSteady: the copies of s+1 .. s+kStages-1 are in flight; otherwise `ahead` stages after s+1 are.
         // FP8: a stage is a single k-step, so the hand-over comes first and the register sets alternate by stage:
         // MFMAs of stage s run on set s % 2 while stage s+1 is read into the other set.
-        auto run_stage = [&](int s, auto steady_tag, int ahead, bool next, auto odd_tag) {
+        // copies c with slot_lo(t) <= c < slot_lo(t + 1) go out behind MFMA t: n copies spread evenly over the NM slots
+        // (the texture path moves one 1 KiB copy per 16 cycles for the whole CU; bunched copies back up into the
+        // issue queues of all four wavefronts)
+        auto run_stage = [&](int s, auto steady_tag, int ahead, bool next, bool deferred, auto odd_tag) {
             constexpr bool kSteady = decltype(steady_tag)::value;
             constexpr int kCur = FP8 ? (decltype(odd_tag)::value ? 1 : 0) : 1;   // set used by the MFMAs after the hand-over
+            constexpr int kFirst = FP8 ? kLoads : kLoads / 2;   // copies of stage s + kStages issued in this stage
+            constexpr int kLate = kLoads - kFirst;              // ... and behind the first MFMAs of the next stage
             if constexpr (!FP8) {
 #pragma unroll
                 for (int t = 0; t < NM; ++t) {
                     mfma_one(0, t);
                     if (t < NR) load_frag(s, 1, 1, t);
+                    if (deferred) {
+#pragma unroll
+                        for (int c = t * kLate / NM; c < (t + 1) * kLate / NM; ++c) issue_copy(s - 1 + kStages, kFirst + c);
+                    }
                     __builtin_amdgcn_sched_barrier(0);
                 }
             }
@@ -298,56 +337,52 @@ void gmm_direct_kernel(const GmmArgs p) {
                 // 8 registers per operand: A fragments live in one register set and are re-read for stage s+1
                 // right behind their last MFMA of this stage; B fragments alternate between two sets.
 #pragma unroll
-                for (int t = 0; t < (NM > FN + kLoads ? NM : FN + kLoads); ++t) {
-                    if (t < NM) mfma_one_fp8(kCur, t);
+                for (int t = 0; t < NM; ++t) {
+                    mfma_one_fp8(kCur, t);
                     if (kSteady || next) {
                         if (t < FN) load_frag(s + 1, 0, kCur ^ 1, FM + t);
-                        else if (kSteady && t < FN + kLoads) issue_copy(s + kStages, t - FN);
-                        if (t < NM && (t % FN) == FN - 1) load_frag(s + 1, 0, 0, t / FN);
+                        if ((t % FN) == FN - 1) load_frag(s + 1, 0, 0, t / FN);
+                    }
+                    if constexpr (kSteady) {
+#pragma unroll
+                        for (int c = t * kFirst / NM; c < (t + 1) * kFirst / NM; ++c) issue_copy(s + kStages, c);
                     }
                     __builtin_amdgcn_sched_barrier(0);
                 }
             } else {
 #pragma unroll
-                for (int t = 0; t < (NM > NR + kLoads ? NM : NR + kLoads); ++t) {
-                    if (t < NM) mfma_one(kCur, t);
-                    if (kSteady || next) {
-                        if (t < NR) load_frag(s + 1, 0, kCur ^ 1, t);
-                        else if (kSteady && t < NR + kLoads) issue_copy(s + kStages, t - NR);
+                for (int t = 0; t < NM; ++t) {
+                    mfma_one(kCur, t);
+                    if ((kSteady || next) && t < NR) load_frag(s + 1, 0, kCur ^ 1, t);
+                    if constexpr (kSteady) {
+#pragma unroll
+                        for (int c = t * kFirst / NM; c < (t + 1) * kFirst / NM; ++c) issue_copy(s + kStages, c);
                     }
                     __builtin_amdgcn_sched_barrier(0);
                 }
             }
         };
-        auto step = [&](int s, auto steady_tag, int ahead, bool next) {
-            if (FP8 && (s & 1)) run_stage(s, steady_tag, ahead, next, std::true_type{});
-            else run_stage(s, steady_tag, ahead, next, std::false_type{});
+        auto step = [&](int s, auto steady_tag, int ahead, bool next, bool deferred) {
+            if (FP8 && (s & 1)) run_stage(s, steady_tag, ahead, next, deferred, std::true_type{});
+            else run_stage(s, steady_tag, ahead, next, deferred, std::false_type{});
         };
         int s = 0;
         if constexpr (FP8) {
             // even and odd stages as one straight-line loop body: the accumulators stay where they are
             for (; s + 1 + kStages < S; s += 2) {
-                run_stage(s, std::true_type{}, 0, true, std::false_type{});
-                run_stage(s + 1, std::true_type{}, 0, true, std::true_type{});
+                run_stage(s, std::true_type{}, 0, true, false, std::false_type{});
+                run_stage(s + 1, std::true_type{}, 0, true, false, std::true_type{});
             }
         }
-        for (; s + kStages < S; ++s) step(s, std::true_type{}, 0, true);
+        // bf16: the second half of a stage's copies goes out one stage later, behind the MFMAs of k-step 0; the first
+        // stage after the steady ones still owes the late copies of the last steady stage
+        for (; s + kStages < S; ++s) step(s, std::true_type{}, 0, true, !FP8 && s > 0);
         for (; s < S; ++s) {
             const int left = S - 1 - s;                           // stages after this one
-            step(s, std::false_type{}, left - 1 < kStages - 2 ? left - 1 : kStages - 2, left > 0);
+            step(s, std::false_type{}, left - 1 < kStages - 2 ? left - 1 : kStages - 2, left > 0,
+                 !FP8 && s > 0 && s + kStages == S);
         }
 
-        auto next_item = [&]() {
-            // ---- next work item and its first copies ----
-            if (tid == 0) s_item = sched_item(draw, streams);
-            __syncthreads();   // also: the last stage has been read by everyone, LDS may be refilled
-            q = s_item;
-            if (q < total) {
-                if (tid == 0) draw = sched_draw(p.sched_slot, streams);
-                open_tile(q);
-                issue_prologue();
-            }
-        };
         auto epilogue = [&]() {
             // ---- epilogue of the finished tile ----
             // The MFMAs take the B fragment as their first operand, so an accumulator holds the tile transposed:
@@ -404,15 +439,26 @@ void gmm_direct_kernel(const GmmArgs p) {
     
         };
 #ifdef DMOE_DEBUG_HOOKS
-        // timing experiments: 5 = the next tile's first copies go out before the results are stored; 6 = results not stored
-        if (p.dbg == 5) { next_item(); epilogue(); }
-        else if (p.dbg == 6) { next_item(); }
-        else { epilogue(); next_item(); }
-#else
-        // stores first: they are then older than the next tile's copies and never hold up a vmcnt wait of its pipeline
-        epilogue();
-        next_item();
+        if (p.dbg == 6) return;   // timing experiment: results not stored
 #endif
+        epilogue();
+        };   // run_tile
+        if (nfr == FM) run_tile(std::false_type{});
+        else run_tile(std::true_type{});
+
+        auto next_item = [&]() {
+            // ---- next work item and its first copies ----
+            if (tid == 0) s_item = sched_item(draw, streams);
+            __syncthreads();   // also: the last stage has been read by everyone, LDS may be refilled
+            q = s_item;
+            if (q < total) {
+                if (tid == 0) draw = sched_draw(p.sched_slot, streams);
+                open_tile(q);
+                issue_prologue();
+            }
+        };
+        // stores first: they are then older than the next tile's copies and never hold up a vmcnt wait of its pipeline
+        next_item();
     }
     sched_finish(p.sched_slot);
 }

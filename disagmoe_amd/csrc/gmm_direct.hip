@@ -24,15 +24,33 @@ typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef short s16x8 __attribute__((ext_vector_type(8)));
 #define DMOE_LDS_PTR(p) ((__attribute__((address_space(3))) void *)(p))
 
-// One wavefront copies 64 x 16 bytes from per-lane global addresses to 1 KiB of LDS at `lds`
-// (wave-uniform byte address, goes through M0).  Written as asm so that the compiler does not
-// serialise later LDS reads behind every outstanding copy; completion is tracked by hand
-// with vmcnt (the copies complete in issue order).
-__device__ __forceinline__ void copy_g2lds_16(const char *gptr, uint32_t lds) {
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
-                 :: "v"(gptr), "s"(__builtin_amdgcn_readfirstlane(lds)) : "memory", "m0");
+// One wavefront copies 64 x 16 bytes from global memory to 1 KiB of LDS.  Lane l reads at base + off (wave-uniform
+// 64-bit base in scalar registers, 32-bit unsigned lane offset) and its bytes land at lds + kLdsImm + 16 l (wave-uniform
+// byte address, goes through M0).  Three instructions; written as asm so that the compiler does not serialise later
+// LDS reads behind every outstanding copy: completion is tracked by hand with vmcnt (the copies complete in issue order).
+template <int kLdsImm>
+__device__ __forceinline__ void copy_g2lds_16(uint32_t off, uint64_t base, uint32_t lds) {
+    asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :: "v"(off), "s"(base), "s"(lds), "n"(kLdsImm) : "memory", "m0", "scc");
+}
+// a wave-uniform 64-bit value held in a VGPR pair, moved to scalar registers
+__device__ __forceinline__ uint64_t to_scalar(uint64_t v) {
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return ((uint64_t)hi << 32) | lo;
 }
 __device__ __forceinline__ uint32_t lds_addr(const void *p) { return (uint32_t)(uintptr_t)DMOE_LDS_PTR(p); }
+
+// f(integral_constant<int, I>) for I = LO .. HI-1, unrolled at compile time
+template <int LO, int HI, typename F>
+__device__ __forceinline__ void static_for(F &&f) {
+    if constexpr (LO < HI) {
+        f(std::integral_constant<int, LO>{});
+        static_for<LO + 1, HI>(f);
+    }
+}
+// n copies spread evenly over the MFMA slots first .. slots-1 of a k-step: the copies behind MFMA t are
+// copy_slot(t) .. copy_slot(t + 1) - 1
+constexpr int copy_slot(int t, int n, int first, int slots) { return t < first ? 0 : (t - first) * n / (slots - first); }
 
 constexpr int kDN = 256;                   // tile columns
 constexpr int kDK = 32;                    // k per stage
@@ -102,8 +120,8 @@ void gmm_direct_kernel(const GmmArgs p) {
 
     // ---- state of the tile whose copies are being issued (set by open_tile) ----
     int e = 0, row0 = 0, rows_e = 0, n0 = 0;
-    const char *a_base = nullptr, *b_exp = nullptr;
-    uint32_t a_off[CA], b_off[4];
+    uint64_t a_base = 0, b_exp = 0;      // wave-uniform bases of the tile's rows of a and of the expert's weights
+    uint32_t a_off[CA], b_off[4];        // per-lane byte offsets of this wavefront's copies from those bases
 
     // tile column slot (0..255) -> column of b; slots past the end read the first column (never stored)
     auto b_col = [&](int slot) {
@@ -119,67 +137,45 @@ void gmm_direct_kernel(const GmmArgs p) {
     auto open_tile = [&](long long q) {
         const TileCoord tc = decode_tile<kDM>(q, G, total, n_tiles, E, s_tile_start, s_row_start);
         e = tc.e; row0 = tc.row0; rows_e = tc.rows_e; n0 = tc.nt * BNO;
-        a_base = p.a + (long long)row0 * pitch;
-        b_exp = p.b + (long long)e * p.K * p.N * (FP8 ? 1 : 2);
+        a_base = to_scalar((uint64_t)(uintptr_t)p.a + (uint64_t)row0 * pitch);
+        b_exp = to_scalar((uint64_t)(uintptr_t)p.b + (uint64_t)e * p.K * p.N * (FP8 ? 1 : 2));
 #pragma unroll
         for (int i = 0; i < CA; ++i) {
             int r = (i * 4 + wave) * 16 + kc_row;
             if (r >= rows_e) r = rows_e - 1;                   // clamp: loaded, never stored
             a_off[i] = (uint32_t)r * pitch + kc_chunk * 16;
-#ifdef DMOE_DEBUG_HOOKS
-            // timing experiment 8 (wrong results): whole 128-byte lines, 8 rows per copy, the other 8 rows on odd stages
-            if (p.dbg == 8) a_off[i] = (uint32_t)((i * 4 + wave) * 16 + (lane >> 3)) * pitch + (lane & 7) * 16;
-#endif
         }
         if constexpr (TRANS_B) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) b_off[i] = (uint32_t)b_col((i * 4 + wave) * 16 + kc_row) * pitch + kc_chunk * 16;
-#ifdef DMOE_DEBUG_HOOKS
-            if (p.dbg == 8) {
+        } else {
+            // block i of this wavefront holds k-rows 8 i + kn_k of the stage
 #pragma unroll
-                for (int i = 0; i < 4; ++i) b_off[i] = (uint32_t)b_col((i * 4 + wave) * 16 + (lane >> 3)) * pitch + (lane & 7) * 16;
-            }
-#endif
+            for (int i = 0; i < 4; ++i)
+                b_off[i] = (uint32_t)(i * 8 + kn_k) * (uint32_t)p.N * 2 + (uint32_t)b_col(kn_chunk * 8) * 2;
         }
-        if constexpr (!TRANS_B) b_off[0] = (uint32_t)kn_k * (uint32_t)p.N * 2 + (uint32_t)b_col(kn_chunk * 8) * 2;
     };
 
     // copy number c (0 .. kLoads-1) of this wavefront for stage s: first its CA blocks of A, then its 4 blocks of B
-    auto issue_copy = [&](int s, int c) {
+    auto issue_copy = [&](int s, auto c_tag) {
+        constexpr int c = decltype(c_tag)::value;
 #ifdef DMOE_DEBUG_HOOKS
         // timing experiments (wrong results): 1 = no copies after the prologue, 2 = no A copies, 3 = no B copies
         if (s >= kStages && (p.dbg == 1 || (p.dbg == 2 && c < CA) || (p.dbg == 3 && c >= CA))) return;
 #endif
-        const uint32_t lA = smem_addr + (s % kStages) * kStage + wave * 1024;
-#ifdef DMOE_DEBUG_HOOKS
-        if (p.dbg == 9) {   // timing experiment (wrong results): every stage fetches the bytes of stage 0 again
-            const uint32_t lA9 = smem_addr + (s % kStages) * kStage + wave * 1024;
-            if (c < CA) copy_g2lds_16(a_base + a_off[c], lA9 + c * 4096);
-            else if constexpr (TRANS_B) copy_g2lds_16(b_exp + b_off[c - CA], lA9 + kStageA + (c - CA) * 4096);
-            else copy_g2lds_16(b_exp + ((long long)(c - CA) * 8) * p.N * 2 + b_off[0], lA9 + kStageA + (c - CA) * 4096);
-            return;
-        }
-        if (p.dbg == 8 && TRANS_B) {
-            const long long line = (long long)(s >> 1) * 128 + (long long)(s & 1) * 8 * pitch;
-            if (c < CA) copy_g2lds_16(a_base + line + a_off[c], lA + c * 4096);
-            else copy_g2lds_16(b_exp + line + b_off[c - CA], lA + kStageA + (c - CA) * 4096);
-            return;
-        }
-#endif
-        if (c < CA) {
-            copy_g2lds_16(a_base + (long long)s * 64 + a_off[c], lA + c * 4096);
+        const uint32_t lds = smem_addr + (s % kStages) * kStage + wave * 1024;
+        if constexpr (c < CA) {
+            copy_g2lds_16<c * 4096>(a_off[c], a_base + (uint64_t)s * 64, lds);
         } else {
-            const int i = c - CA;
-            const uint32_t lB = lA + kStageA + i * 4096;
-            if constexpr (TRANS_B) copy_g2lds_16(b_exp + (long long)s * 64 + b_off[i], lB);
-            else copy_g2lds_16(b_exp + ((long long)s * kDK + i * 8) * p.N * 2 + b_off[0], lB);
+            constexpr int i = c - CA;
+            if constexpr (TRANS_B) copy_g2lds_16<kStageA + i * 4096>(b_off[i], b_exp + (uint64_t)s * 64, lds);
+            else copy_g2lds_16<kStageA + i * 4096>(b_off[i], b_exp + (uint64_t)s * kDK * p.N * 2, lds);
         }
     };
     const int pre = S < kStages ? S : kStages;      // stages whose copies are issued ahead of the tile's first MFMA
     auto issue_prologue = [&]() {
         for (int s = 0; s < pre; ++s) {
-#pragma unroll
-            for (int c = 0; c < kLoads; ++c) issue_copy(s, c);
+            static_for<0, kLoads>([&](auto c) { issue_copy(s, c); });
         }
     };
 
@@ -314,53 +310,51 @@ void gmm_direct_kernel(const GmmArgs p) {
             constexpr bool kSteady = decltype(steady_tag)::value;
             constexpr int kCur = FP8 ? (decltype(odd_tag)::value ? 1 : 0) : 1;   // set used by the MFMAs after the hand-over
             constexpr int kFirst = FP8 ? kLoads : kLoads / 2;   // copies of stage s + kStages issued in this stage
-            constexpr int kLate = kLoads - kFirst;              // ... and behind the first MFMAs of the next stage
+            constexpr int kLate = kLoads - kFirst;              // ... and behind the MFMAs of k-step 0 of the next stage
+            // bf16: copies go behind the MFMAs that have no operand read if those slots suffice
+            constexpr int kSlot0 = FP8 ? 0 : (NM - NR >= kLate ? NR : 0);
             if constexpr (!FP8) {
-#pragma unroll
-                for (int t = 0; t < NM; ++t) {
+                static_for<0, NM>([&](auto t_tag) {
+                    constexpr int t = decltype(t_tag)::value;
                     mfma_one(0, t);
                     if (t < NR) load_frag(s, 1, 1, t);
                     if (deferred) {
-#pragma unroll
-                        for (int c = t * kLate / NM; c < (t + 1) * kLate / NM; ++c) issue_copy(s - 1 + kStages, kFirst + c);
+                        static_for<copy_slot(t, kLate, kSlot0, NM), copy_slot(t + 1, kLate, kSlot0, NM)>(
+                            [&](auto c) { issue_copy(s - 1 + kStages, std::integral_constant<int, kFirst + decltype(c)::value>{}); });
                     }
                     __builtin_amdgcn_sched_barrier(0);
-                }
+                });
             }
             if (kSteady || next) {
+#ifdef DMOE_DEBUG_HOOKS
+                if (kSteady && p.dbg == 13) {}   // timing experiment (wrong results): no wait for the copies
+                else
+#endif
                 if constexpr (kSteady) DMOE_WAIT_VMCNT((kStages - 2) * kLoads);
                 else wait_ahead(ahead);
                 __syncthreads();
                 __builtin_amdgcn_sched_barrier(0);
             }
-            if constexpr (FP8) {
-                // 8 registers per operand: A fragments live in one register set and are re-read for stage s+1
-                // right behind their last MFMA of this stage; B fragments alternate between two sets.
-#pragma unroll
-                for (int t = 0; t < NM; ++t) {
+            static_for<0, NM>([&](auto t_tag) {
+                constexpr int t = decltype(t_tag)::value;
+                if constexpr (FP8) {
+                    // 8 registers per operand: A fragments live in one register set and are re-read for stage s+1
+                    // right behind their last MFMA of this stage; B fragments alternate between two sets.
                     mfma_one_fp8(kCur, t);
                     if (kSteady || next) {
                         if (t < FN) load_frag(s + 1, 0, kCur ^ 1, FM + t);
                         if ((t % FN) == FN - 1) load_frag(s + 1, 0, 0, t / FN);
                     }
-                    if constexpr (kSteady) {
-#pragma unroll
-                        for (int c = t * kFirst / NM; c < (t + 1) * kFirst / NM; ++c) issue_copy(s + kStages, c);
-                    }
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-            } else {
-#pragma unroll
-                for (int t = 0; t < NM; ++t) {
+                } else {
                     mfma_one(kCur, t);
                     if ((kSteady || next) && t < NR) load_frag(s + 1, 0, kCur ^ 1, t);
-                    if constexpr (kSteady) {
-#pragma unroll
-                        for (int c = t * kFirst / NM; c < (t + 1) * kFirst / NM; ++c) issue_copy(s + kStages, c);
-                    }
-                    __builtin_amdgcn_sched_barrier(0);
                 }
-            }
+                if constexpr (kSteady) {
+                    static_for<copy_slot(t, kFirst, kSlot0, NM), copy_slot(t + 1, kFirst, kSlot0, NM)>(
+                        [&](auto c) { issue_copy(s + kStages, c); });
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            });
         };
         auto step = [&](int s, auto steady_tag, int ahead, bool next, bool deferred) {
             if (FP8 && (s & 1)) run_stage(s, steady_tag, ahead, next, deferred, std::true_type{});

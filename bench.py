@@ -168,16 +168,23 @@ def main() -> int:
         q_ms, _ = _event_ms(lambda: gg.quantize_rows(permuted), it)
         stages["quant_rows"] = {"ms": q_ms}
         peak = PEAK_FP8_TFLOPS
-        kernel = "dmoe::gmm_kernel<.., swiglu, fp8> (gate-up projection with fused SiLU*mul)"
+        avg = w.R // w.E
+        tile = 64 if avg <= 64 else (128 if avg <= 160 else 256)
+        # mirrors the dispatch of launch_by_rows (csrc/gmm.hip): the fused fp8 gate-up projection on 256-row tiles
+        # runs on the register-staged kernel, every other case on the global-to-LDS kernel
+        kernel = ("dmoe::gmm_kernel<256, 256, .., swiglu, fp8>" if tile == 256 or w.d % 64 or w.d < 448
+                  else f"dmoe::gmm_direct_kernel<{tile}, .., swiglu, fp8>") + " (gate-up projection with fused SiLU*mul)"
     else:
         h = gg.gmm_swiglu(permuted, layer.w13_weight, batch_sizes)
         up_ms, _ = _event_ms(lambda: gg.gmm_swiglu(permuted, layer.w13_weight, batch_sizes, c=h), it)
         y_buf = torch.empty((w.R, w.d), dtype=torch.bfloat16, device=dev)
         down_ms, _ = _event_ms(lambda: gg.gmm(h, layer.w2_weight, batch_sizes, c=y_buf), it)
         peak = PEAK_BF16_TFLOPS
-        big = w.R // w.E > 160 and w.d % 32 == 0
-        kernel = ("dmoe::gmm_direct_kernel<false, true>" if big else "dmoe::gmm_kernel<.., swiglu, bf16>") + \
-            " (gate-up projection with fused SiLU*mul)"
+        avg = w.R // w.E
+        tile = 64 if avg <= 64 else (128 if avg <= 160 else 256)
+        direct = w.d % 32 == 0 and w.d >= 224
+        kernel = (f"dmoe::gmm_direct_kernel<{tile}, .., [K,N] weights, swiglu, bf16>" if direct
+                  else f"dmoe::gmm_kernel<{tile}, 256, .., swiglu, bf16>") + " (gate-up projection with fused SiLU*mul)"
     up_flops = 2.0 * w.R * w.d * 2 * w.I
     down_flops = 2.0 * w.R * w.I * w.d
     stages["gemm_gate_up"] = {"ms": up_ms, "TFLOP/s": up_flops / up_ms / 1e9, "frac_mfma": up_flops / up_ms / 1e9 / peak}

@@ -441,13 +441,12 @@ static int launch_by_rows(const GmmArgs &args, hipStream_t stream) {
     const int tile_rows = avg <= 64 ? 64 : (avg <= 160 ? 128 : 256);
     if constexpr (!FP8) {
         // global -> LDS direct path: whole stages of 32 k, 32-bit offsets inside one expert's weights
-        // (more stages than LDS buffers: K >= 7 * 32 covers every tile size)
-        if (args.K % 32 == 0 && args.K >= 224 && (long long)args.K * args.N * 2 < (1ll << 32))
+        if (args.K % 32 == 0 && (long long)args.K * args.N * 2 < (1ll << 32))
             return launch_direct_bf16(args, tile_rows, TRANS_B, SWIGLU, stream);
     } else {
         // measured on the 8x22b shapes: with 256-row tiles the register-staged 8-wave kernel is ahead for the fused
         // gate-up projection, the direct kernel (128-row tiles at most) for the plain product
-        if (args.K % 64 == 0 && args.K >= 448 && (long long)args.K * args.N < (1ll << 32) && !(SWIGLU && tile_rows == 256))
+        if (args.K % 64 == 0 && (long long)args.K * args.N < (1ll << 32) && !(SWIGLU && tile_rows == 256))
             return launch_direct_fp8(args, tile_rows, SWIGLU, stream);
     }
     if (tile_rows == 64) return launch_one<64, 256, 1, 4, TRANS_B, SWIGLU, FP8>(args, stream);

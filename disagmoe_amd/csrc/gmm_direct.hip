@@ -156,15 +156,14 @@ void gmm_direct_kernel(const GmmArgs p) {
         }
     };
 
-    // copy number c (0 .. kLoads-1) of this wavefront for stage s of the tile described by a_base / b_exp / a_off /
-    // b_off into LDS buffer `buf`: first its CA blocks of A, then its 4 blocks of B
-    auto issue_copy = [&](int buf, int s, auto c_tag) {
+    // copy number c (0 .. kLoads-1) of this wavefront for stage s: first its CA blocks of A, then its 4 blocks of B
+    auto issue_copy = [&](int s, auto c_tag) {
         constexpr int c = decltype(c_tag)::value;
 #ifdef DMOE_DEBUG_HOOKS
         // timing experiments (wrong results): 1 = no copies after the prologue, 2 = no A copies, 3 = no B copies
-        if (p.dbg == 1 || (p.dbg == 2 && c < CA) || (p.dbg == 3 && c >= CA)) return;
+        if (s >= kStages && (p.dbg == 1 || (p.dbg == 2 && c < CA) || (p.dbg == 3 && c >= CA))) return;
 #endif
-        const uint32_t lds = smem_addr + buf * kStage + wave * 1024;
+        const uint32_t lds = smem_addr + (s % kStages) * kStage + wave * 1024;
         if constexpr (c < CA) {
             copy_g2lds_16<c * 4096>(a_off[c], a_base + (uint64_t)s * 64, lds);
         } else {
@@ -173,13 +172,12 @@ void gmm_direct_kernel(const GmmArgs p) {
             else copy_g2lds_16<kStageA + i * 4096>(b_off[i], b_exp + (uint64_t)s * kDK * p.N * 2, lds);
         }
     };
-    // the first kStages stages of a workgroup's first tile go out at once (S > kStages is a launch precondition)
+    const int pre = S < kStages ? S : kStages;      // stages whose copies are issued ahead of the tile's first MFMA
     auto issue_prologue = [&]() {
-        for (int s = 0; s < kStages; ++s) {
-            static_for<0, kLoads>([&](auto c) { issue_copy(s, s, c); });
+        for (int s = 0; s < pre; ++s) {
+            static_for<0, kLoads>([&](auto c) { issue_copy(s, c); });
         }
     };
-    auto wrap = [](int b) { return b >= kStages ? b - kStages : b; };   // LDS buffer index after an increment
 
     // B operand rows / columns of this wavefront: fragment j covers 32 tile columns
     int fb_off[FN];
@@ -198,10 +196,10 @@ void gmm_direct_kernel(const GmmArgs p) {
 
     typedef typename std::conditional<FP8, i32x8, bf16x8>::type frag_t;
     frag_t fa[FP8 ? 1 : 2][FM], fb[2][FN];
-    // operand read number r (0 .. NR-1) of k-step ks of the stage in LDS buffer `buf` into register set `slot`: first
-    // the FM A fragments, then the FN B fragments
-    auto load_frag = [&](int buf, int ks, int slot, int r) {
-        const char *tA = smem + buf * kStage;
+    // operand read number r (0 .. NR-1) of k-step ks of stage s into register set `slot`: first the FM A fragments,
+    // then the FN B fragments
+    auto load_frag = [&](int s, int ks, int slot, int r) {
+        const char *tA = smem + (s % kStages) * kStage;
         const char *tB = tA + kStageA;
         const int c0 = ((ks * 2 + kgrp) ^ f_sw) << 4;
         if constexpr (FP8) {
@@ -241,10 +239,7 @@ void gmm_direct_kernel(const GmmArgs p) {
         else DMOE_WAIT_VMCNT(0);
     };
 
-    // ---- work items ----
-    // The pipeline does not drain between tiles: while the last kStages stages of a tile are multiplied, the copies
-    // of the next tile's first kStages stages go out in the slots the tile itself no longer needs, and the operand
-    // reads of its stage 0 ride behind the tile's last MFMAs.  Between two tiles there is only the epilogue.
+    // ---- first work item ----
     unsigned int draw = 0;
     if (tid == 0) {
         draw = sched_draw(p.sched_slot, streams);
@@ -253,32 +248,17 @@ void gmm_direct_kernel(const GmmArgs p) {
     }
     __syncthreads();
     long long q = s_item;
-    __syncthreads();                // s_item is rewritten at the start of the first tile
-    int buf0 = 0;                   // LDS buffer of the current tile's stage 0
-    int par0 = 0;                   // fp8: register set of the B fragments of the current tile's stage 0
-    bool fresh = true;              // first tile of the workgroup: filled by the prologue, nothing else in flight
-    bool credit = false;            // this wavefront stored the previous tile with exactly kStores store instructions
     if (q < total) {
         open_tile(q);
         issue_prologue();
     }
-    constexpr int kStores = FM * (SWIGLU ? FN / 2 : FN) * 4;           // stores of a full tile per wavefront
-    constexpr int kNormalWait = (kStages - 2) * kLoads;                // copies younger than stage s+1 at a hand-over
-    constexpr int kCreditWait = kNormalWait + kStores > 63 ? 63 : kNormalWait + kStores;
-    constexpr int kCreditStages = kStages - 2 + (FP8 ? 1 : 0);         // hand-overs that still have the stores behind stage s+1
 
     while (q < total) {
+        // results of this tile go here after the next tile's copies have been issued
         const int cur_row0 = row0, cur_rows_e = rows_e, cur_n0 = n0, cur_e = e;
         // row fragments of this wavefront that hold at least one valid row (a short last tile skips the rest)
         int nfr = ((rows_e < kDM ? rows_e : kDM) - wm * TM + 31) / 32;
         nfr = __builtin_amdgcn_readfirstlane(nfr < 0 ? 0 : (nfr > FM ? FM : nfr));
-        // the item after this one: published here, read behind the first barrier of the tile
-        if (tid == 0) {
-            s_item = sched_item(draw, streams);
-            draw = sched_draw(p.sched_slot, streams);
-        }
-        bool next_credit = false;
-        long long q_next = total;
 
         // The tile from its first MFMA to its last store, in two builds: without any branch around the MFMAs (every
         // row fragment of this wavefront holds rows: all but the last tile of an expert) and with one per MFMA.
@@ -305,46 +285,42 @@ void gmm_direct_kernel(const GmmArgs p) {
                 acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[bslot][j], fa[0][i], acc[i][j], 0, 0, 0, 0, 0, 0);
         };
 
-        if (fresh) {
-            // stage 0 has landed; the other kStages - 1 prologue stages may still be in flight
-            DMOE_WAIT_VMCNT((kStages - 1) * kLoads);
-            __syncthreads();
+        // stage 0 of this tile has landed (its other prologue stages, and stores of the previous tile's
+        // epilogue that were issued after them, may still be in flight: waiting for fewer is only stricter)
+        wait_ahead(pre - 1);
+        __syncthreads();
 #pragma unroll
-            for (int r = 0; r < NR; ++r) load_frag(buf0, 0, 0, r);
-        }
+        for (int r = 0; r < NR; ++r) load_frag(0, 0, 0, r);
 
         // One stage = 2 k-steps of NM MFMAs.  A wavefront issues in order and an MFMA occupies the matrix pipe
-        // for 32 cycles, so the LDS reads and global -> LDS copies are slotted behind MFMAs: they are issued in
+        // for 32 cycles, so the LDS reads and global -> LDS copies are slotted one per MFMA: they are issued in
         // the shadow of the MFMA before them and the pipe never waits for the issue port.
-        //   k-step 0: MFMAs on register set 0; the NR operand reads of k-step 1 go to set 1; the late half of the
-        //              copies that refill the buffer of the stage before.
+        //   k-step 0: MFMAs on register set 0; the NR operand reads of k-step 1 go to set 1.
         //   hand-over: this wavefront's share of stage s+1 has landed (vmcnt), barrier (everybody's has, and
         //              every read of stage s is complete).
-        //   k-step 1: MFMAs on set 1; the NR operand reads of stage s+1 go to set 0; the first half of the copies
-        //              that refill this stage's buffer (with stage s + kStages of this tile, or of the next one).
+        //   k-step 1: MFMAs on set 1; the NR operand reads of stage s+1 go to set 0; the copies that refill the LDS
+        //              stage just drained with stage s + kStages are spread over this k-step and the next one.
         // kSteady: the copies of s+1 .. s+kStages-1 are in flight; otherwise `ahead` stages after s+1 are.
         // FP8: a stage is a single k-step, so the hand-over comes first and the register sets alternate by stage:
-        // MFMAs of a stage run on one B set while the next stage is read into the other; all copies are "first".
-        //   b: LDS buffer of the stage; cs: stage (relative to the tile whose addresses are loaded) that refills it;
-        //   cl: the same for the late copies into the buffer before; switch_to: item whose addresses are loaded at
-        //   the hand-over (-1: none).
-        auto run_stage = [&](int b, int cs, int cl, auto steady_tag, int ahead, bool next, bool deferred, bool use_credit,
-                             long long switch_to, auto odd_tag) {
+        // MFMAs of stage s run on set s % 2 while stage s+1 is read into the other set.
+        // copies c with slot_lo(t) <= c < slot_lo(t + 1) go out behind MFMA t: n copies spread evenly over the NM slots
+        // (the texture path moves one 1 KiB copy per 16 cycles for the whole CU; bunched copies back up into the
+        // issue queues of all four wavefronts)
+        auto run_stage = [&](int s, auto steady_tag, int ahead, bool next, bool deferred, auto odd_tag) {
             constexpr bool kSteady = decltype(steady_tag)::value;
             constexpr int kCur = FP8 ? (decltype(odd_tag)::value ? 1 : 0) : 1;   // set used by the MFMAs after the hand-over
-            constexpr int kFirst = FP8 ? kLoads : kLoads / 2;
-            constexpr int kLate = kLoads - kFirst;
+            constexpr int kFirst = FP8 ? kLoads : kLoads / 2;   // copies of stage s + kStages issued in this stage
+            constexpr int kLate = kLoads - kFirst;              // ... and behind the MFMAs of k-step 0 of the next stage
             // bf16: copies go behind the MFMAs that have no operand read if those slots suffice
             constexpr int kSlot0 = FP8 ? 0 : (NM - NR >= kLate ? NR : 0);
-            const int nb = wrap(b + 1), pb = wrap(b + kStages - 1);
             if constexpr (!FP8) {
                 static_for<0, NM>([&](auto t_tag) {
                     constexpr int t = decltype(t_tag)::value;
                     mfma_one(0, t);
-                    if (t < NR) load_frag(b, 1, 1, t);
+                    if (t < NR) load_frag(s, 1, 1, t);
                     if (deferred) {
                         static_for<copy_slot(t, kLate, kSlot0, NM), copy_slot(t + 1, kLate, kSlot0, NM)>(
-                            [&](auto c) { issue_copy(pb, cl, std::integral_constant<int, kFirst + decltype(c)::value>{}); });
+                            [&](auto c) { issue_copy(s - 1 + kStages, std::integral_constant<int, kFirst + decltype(c)::value>{}); });
                     }
                     __builtin_amdgcn_sched_barrier(0);
                 });
@@ -354,16 +330,11 @@ void gmm_direct_kernel(const GmmArgs p) {
                 if (kSteady && p.dbg == 13) {}   // timing experiment (wrong results): no wait for the copies
                 else
 #endif
-                if constexpr (kSteady) {
-                    if (use_credit) DMOE_WAIT_VMCNT(kCreditWait);
-                    else DMOE_WAIT_VMCNT(kNormalWait);
-                } else {
-                    wait_ahead(ahead);
-                }
+                if constexpr (kSteady) DMOE_WAIT_VMCNT((kStages - 2) * kLoads);
+                else wait_ahead(ahead);
                 __syncthreads();
                 __builtin_amdgcn_sched_barrier(0);
             }
-            if (switch_to >= 0) open_tile(switch_to);
             static_for<0, NM>([&](auto t_tag) {
                 constexpr int t = decltype(t_tag)::value;
                 if constexpr (FP8) {
@@ -371,65 +342,40 @@ void gmm_direct_kernel(const GmmArgs p) {
                     // right behind their last MFMA of this stage; B fragments alternate between two sets.
                     mfma_one_fp8(kCur, t);
                     if (kSteady || next) {
-                        if (t < FN) load_frag(nb, 0, kCur ^ 1, FM + t);
-                        if ((t % FN) == FN - 1) load_frag(nb, 0, 0, t / FN);
+                        if (t < FN) load_frag(s + 1, 0, kCur ^ 1, FM + t);
+                        if ((t % FN) == FN - 1) load_frag(s + 1, 0, 0, t / FN);
                     }
                 } else {
                     mfma_one(kCur, t);
-                    if ((kSteady || next) && t < NR) load_frag(nb, 0, kCur ^ 1, t);
+                    if ((kSteady || next) && t < NR) load_frag(s + 1, 0, kCur ^ 1, t);
                 }
                 if constexpr (kSteady) {
                     static_for<copy_slot(t, kFirst, kSlot0, NM), copy_slot(t + 1, kFirst, kSlot0, NM)>(
-                        [&](auto c) { issue_copy(b, cs, c); });
+                        [&](auto c) { issue_copy(s + kStages, c); });
                 }
                 __builtin_amdgcn_sched_barrier(0);
             });
         };
-        auto step = [&](int b, int odd, int cs, int cl, auto steady_tag, int ahead, bool next, bool deferred, bool use_credit,
-                        long long switch_to) {
-            if (FP8 && odd) run_stage(b, cs, cl, steady_tag, ahead, next, deferred, use_credit, switch_to, std::true_type{});
-            else run_stage(b, cs, cl, steady_tag, ahead, next, deferred, use_credit, switch_to, std::false_type{});
+        auto step = [&](int s, auto steady_tag, int ahead, bool next, bool deferred) {
+            if (FP8 && (s & 1)) run_stage(s, steady_tag, ahead, next, deferred, std::true_type{});
+            else run_stage(s, steady_tag, ahead, next, deferred, std::false_type{});
         };
-        int s = 0, b = buf0;
-        // stages whose buffers are refilled with later stages of this tile
+        int s = 0;
         if constexpr (FP8) {
-            if (par0 && s + kStages < S) {
-                step(b, 1, s + kStages, 0, std::true_type{}, 0, true, false, credit && s < kCreditStages, -1);
-                ++s; b = wrap(b + 1);
-            }
             // even and odd stages as one straight-line loop body: the accumulators stay where they are
             for (; s + 1 + kStages < S; s += 2) {
-                run_stage(b, s + kStages, 0, std::true_type{}, 0, true, false, credit && s < kCreditStages, -1, std::false_type{});
-                b = wrap(b + 1);
-                run_stage(b, s + 1 + kStages, 0, std::true_type{}, 0, true, false, credit && s + 1 < kCreditStages, -1,
-                          std::true_type{});
-                b = wrap(b + 1);
+                run_stage(s, std::true_type{}, 0, true, false, std::false_type{});
+                run_stage(s + 1, std::true_type{}, 0, true, false, std::true_type{});
             }
         }
-        for (; s + kStages < S; ++s) {
-            step(b, (par0 + s) & 1, s + kStages, s - 1 + kStages, std::true_type{}, 0, true, !FP8 && (s > 0 || !fresh),
-                 credit && s < kCreditStages, -1);
-            b = wrap(b + 1);
+        // bf16: the second half of a stage's copies goes out one stage later, behind the MFMAs of k-step 0; the first
+        // stage after the steady ones still owes the late copies of the last steady stage
+        for (; s + kStages < S; ++s) step(s, std::true_type{}, 0, true, !FP8 && s > 0);
+        for (; s < S; ++s) {
+            const int left = S - 1 - s;                           // stages after this one
+            step(s, std::false_type{}, left - 1 < kStages - 2 ? left - 1 : kStages - 2, left > 0,
+                 !FP8 && s > 0 && s + kStages == S);
         }
-        q_next = s_item;   // at least one barrier lies behind its publication (S > kStages)
-        if (q_next < total) {
-            // the last kStages stages: their buffers are refilled with the first stages of the next tile, whose
-            // addresses are loaded at the first of these hand-overs (the late copies before it still belong to this tile)
-            for (; s < S; ++s) {
-                const int j = s + kStages - S;
-                step(b, (par0 + s) & 1, j, j == 0 ? S - 1 : j - 1, std::true_type{}, 0, true, !FP8 && (s > 0 || !fresh),
-                     credit && s < kCreditStages, j == 0 ? q_next : -1);
-                b = wrap(b + 1);
-            }
-        } else {
-            for (; s < S; ++s) {
-                const int left = S - 1 - s;                           // stages after this one
-                step(b, (par0 + s) & 1, 0, S - 1, std::false_type{}, left - 1 < kStages - 2 ? left - 1 : kStages - 2, left > 0,
-                     !FP8 && (s > 0 || !fresh) && s + kStages == S, false, -1);
-                b = wrap(b + 1);
-            }
-        }
-        next_credit = !kGuard && cur_n0 + BNO <= n_out;
 
         auto epilogue = [&]() {
             // ---- epilogue of the finished tile ----
@@ -494,12 +440,19 @@ void gmm_direct_kernel(const GmmArgs p) {
         if (nfr == FM) run_tile(std::false_type{});
         else run_tile(std::true_type{});
 
-        // the next tile's first stages are in flight and its stage 0 operands are in registers
-        buf0 = (buf0 + S) % kStages;
-        par0 = (par0 + S) & 1;
-        fresh = false;
-        credit = next_credit;
-        q = q_next;
+        auto next_item = [&]() {
+            // ---- next work item and its first copies ----
+            if (tid == 0) s_item = sched_item(draw, streams);
+            __syncthreads();   // also: the last stage has been read by everyone, LDS may be refilled
+            q = s_item;
+            if (q < total) {
+                if (tid == 0) draw = sched_draw(p.sched_slot, streams);
+                open_tile(q);
+                issue_prologue();
+            }
+        };
+        // stores first: they are then older than the next tile's copies and never hold up a vmcnt wait of its pipeline
+        next_item();
     }
     sched_finish(p.sched_slot);
 }
@@ -535,7 +488,7 @@ static int launch_direct_tile(const GmmArgs &args, bool trans_b, bool swiglu, hi
     return swiglu ? launch_direct_one<kDM, WM, false, true, false>(args, stream) : launch_direct_one<kDM, WM, false, false, false>(args, stream);
 }
 
-// Preconditions (checked by the caller): bf16, K % 32 == 0, K / 32 > 6, N % 8 == 0, K * N * 2 < 2^32.
+// Preconditions (checked by the caller): bf16, K % 32 == 0, N % 8 == 0, K * N * 2 < 2^32.
 // tile_rows: 256, 128 or 64.
 int launch_direct_bf16(const GmmArgs &args, int tile_rows, bool trans_b, bool swiglu, hipStream_t stream) {
     if (tile_rows == 64) return launch_direct_tile<64, 1>(args, trans_b, swiglu, stream);
@@ -543,7 +496,7 @@ int launch_direct_bf16(const GmmArgs &args, int tile_rows, bool trans_b, bool sw
     return launch_direct_tile<256, 2>(args, trans_b, swiglu, stream);
 }
 
-// Preconditions: e4m3 operands, K-contiguous on both sides, K % 64 == 0, K / 64 > 6, N % 8 == 0, K * N < 2^32.
+// Preconditions: e4m3 operands, K-contiguous on both sides, K % 64 == 0, N % 8 == 0, K * N < 2^32.
 int launch_direct_fp8(const GmmArgs &args, int tile_rows, bool swiglu, hipStream_t stream) {
     if (tile_rows == 64) return swiglu ? launch_direct_one<64, 1, true, true, true>(args, stream) : launch_direct_one<64, 1, true, false, true>(args, stream);
     // 256-row tiles would need 256 accumulator + 96 operand registers per lane plus addressing: they are cut in two

@@ -51,6 +51,10 @@ __device__ __forceinline__ void static_for(F &&f) {
 // n copies spread evenly over the MFMA slots first .. slots-1 of a k-step: the copies behind MFMA t are
 // copy_slot(t) .. copy_slot(t + 1) - 1
 constexpr int copy_slot(int t, int n, int first, int slots) { return t < first ? 0 : (t - first) * n / (slots - first); }
+// fp8 (all copies of a stage go out in one k-step): MFMA slot behind which copy j of n goes out for the wavefront
+// with number `phase`.  The copies of one wavefront are slots / n apart and the four wavefronts start one slot
+// after each other, so that they do not queue up at the texture path behind the same MFMA.
+constexpr int copy_slot_of(int j, int n, int slots, int phase) { return (j * (slots / n > 0 ? slots / n : 1) + phase) % slots; }
 
 constexpr int kDN = 256;                   // tile columns
 constexpr int kDK = 32;                    // k per stage
@@ -263,7 +267,7 @@ void gmm_direct_kernel(const GmmArgs p) {
         // The tile from its first MFMA to its last store, in two builds: without any branch around the MFMAs (every
         // row fragment of this wavefront holds rows: all but the last tile of an expert) and with one per MFMA.
         // Wavefronts of one workgroup may take different builds; both execute the same copies and barriers.
-        auto run_tile = [&](auto guard_tag) {
+        auto run_tile = [&](auto guard_tag, auto phase_tag) {
         constexpr bool kGuard = decltype(guard_tag)::value;
         f32x16 acc[FM][FN];
 #pragma unroll
@@ -350,8 +354,15 @@ void gmm_direct_kernel(const GmmArgs p) {
                     if ((kSteady || next) && t < NR) load_frag(s + 1, 0, kCur ^ 1, t);
                 }
                 if constexpr (kSteady) {
-                    static_for<copy_slot(t, kFirst, kSlot0, NM), copy_slot(t + 1, kFirst, kSlot0, NM)>(
-                        [&](auto c) { issue_copy(s + kStages, c); });
+                    if constexpr (FP8) {
+                        static_for<0, kFirst>([&](auto c) {
+                            if constexpr (copy_slot_of(decltype(c)::value, kFirst, NM, decltype(phase_tag)::value) == t)
+                                issue_copy(s + kStages, c);
+                        });
+                    } else {
+                        static_for<copy_slot(t, kFirst, kSlot0, NM), copy_slot(t + 1, kFirst, kSlot0, NM)>(
+                            [&](auto c) { issue_copy(s + kStages, c); });
+                    }
                 }
                 __builtin_amdgcn_sched_barrier(0);
             });
@@ -437,8 +448,19 @@ void gmm_direct_kernel(const GmmArgs p) {
 #endif
         epilogue();
         };   // run_tile
-        if (nfr == FM) run_tile(std::false_type{});
-        else run_tile(std::true_type{});
+        // fp8: one instance per wavefront number (the MFMA slots of its copies are compile-time constants)
+        auto run_build = [&](auto guard_tag) {
+            if constexpr (FP8) {
+                if (wave == 0) run_tile(guard_tag, std::integral_constant<int, 0>{});
+                else if (wave == 1) run_tile(guard_tag, std::integral_constant<int, 1>{});
+                else if (wave == 2) run_tile(guard_tag, std::integral_constant<int, 2>{});
+                else run_tile(guard_tag, std::integral_constant<int, 3>{});
+            } else {
+                run_tile(guard_tag, std::integral_constant<int, 0>{});
+            }
+        };
+        if (nfr == FM) run_build(std::false_type{});
+        else run_build(std::true_type{});
 
         auto next_item = [&]() {
             // ---- next work item and its first copies ----

@@ -37,6 +37,10 @@ int fail(int code, const char *fmt, ...);
 
 int device_cus();  // compute units of the current device, cached per device
 
+// True the first time it is called with `seen` on the current device (a function attribute such as the dynamic
+// LDS size is set per device).
+bool first_on_device(unsigned long long *seen);
+
 __device__ __forceinline__ int lane_id() { return threadIdx.x & (kWave - 1); }
 
 // bf16 <-> fp32, round to nearest even (NaN kept quiet).

@@ -399,11 +399,9 @@ static int launch_one(const GmmArgs &args, hipStream_t stream) {
     constexpr int BNO = SWIGLU ? BN / 2 : BN;
     const size_t lds = 2 * (size_t)(BM + BN) * kRowBytes;
     auto kern = gmm_kernel<BM, BN, WM, WN, TRANS_B, SWIGLU, FP8>;
-    static bool configured = false;  // the attribute is per function, not per device context switch
-    if (!configured) {
+    static unsigned long long configured = 0;   // devices on which the kernel's LDS size has been raised
+    if (first_on_device(&configured))
         DMOE_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        configured = true;
-    }
     const int n_out = SWIGLU ? args.N / 2 : args.N;
     const long long n_tiles = (n_out + BNO - 1) / BNO;
     const long long m_tiles_max = args.rows / BM + args.E;  // sum of ceil(n_e / BM) never exceeds this

@@ -485,11 +485,9 @@ static int launch_direct_one(const GmmArgs &args, hipStream_t stream) {
     constexpr int kStages = kDM == 256 ? 4 : (kDM == 128 ? 5 : 6);
     const size_t lds = (size_t)kStages * (kDM * kDK * 2 + kStageB);
     auto kern = gmm_direct_kernel<kDM, WM, TRANS_B, SWIGLU, FP8>;
-    static bool configured = false;
-    if (!configured) {
+    static unsigned long long configured = 0;   // devices on which the kernel's LDS size has been raised
+    if (first_on_device(&configured))
         DMOE_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        configured = true;
-    }
     const int n_out = SWIGLU ? args.N / 2 : args.N;
     const long long n_tiles = (n_out + BNO - 1) / BNO;
     const long long m_tiles_max = args.rows / kDM + args.E;

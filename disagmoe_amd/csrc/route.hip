@@ -40,6 +40,14 @@ int device_cus() {
     return cached[dev];
 }
 
+bool first_on_device(unsigned long long *seen) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return true;
+    const unsigned long long bit = 1ull << (dev & 63);
+    const unsigned long long before = __atomic_fetch_or(seen, bit, __ATOMIC_RELAXED);
+    return (before & bit) == 0;
+}
+
 constexpr int kChunk = 512;       // rows per wavefront
 constexpr int kMaxExperts = 4096; // 3 int tables of E entries must fit in LDS
 

@@ -437,7 +437,7 @@ static int launch_by_rows(const GmmArgs &args, hipStream_t stream) {
         default: break;
     }
     int tile_rows = avg <= 64 ? 64 : (avg <= 160 ? 128 : 256);
-    if (g_variant >= 5) tile_rows = g_variant == 5 ? 64 : (g_variant == 6 ? 128 : 256);   // direct kernel, fixed tile rows
+    if (g_variant >= 5) tile_rows = g_variant == 5 ? 64 : (g_variant == 6 ? 128 : (g_variant == 7 ? 256 : 260));   // direct kernel, fixed tile rows (260: 256 rows on 4 wavefronts)
     if constexpr (!FP8) {
         // global -> LDS direct path: whole stages of 32 k, 32-bit offsets inside one expert's weights
         if (args.K % 32 == 0 && (long long)args.K * args.N * 2 < (1ll << 32))
@@ -474,7 +474,7 @@ extern "C" int dmoe_gmm_tune(int variant) {
 #ifdef DMOE_DEBUG_HOOKS
     if (variant >= 100) { g_debug_mode = variant - 100; return DMOE_OK; }
 #endif
-    DMOE_REQUIRE(variant >= 0 && variant <= 7, DMOE_ERR_ARG, "dmoe_gmm_tune: variant %d outside [0, 7]", variant);
+    DMOE_REQUIRE(variant >= 0 && variant <= 8, DMOE_ERR_ARG, "dmoe_gmm_tune: variant %d outside [0, 8]", variant);
     g_variant = variant;
     return DMOE_OK;
 }

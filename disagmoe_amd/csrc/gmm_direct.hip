@@ -65,24 +65,28 @@ constexpr int kStageB = kDN * kDK * 2;     // 16 KiB of B per stage
 
 // FP8: operands are e4m3 bytes, K-contiguous on both sides (TRANS_B), a stage holds 64 k = one
 // v_mfma_f32_32x32x64_f8f6f4 k-step, and per-row / per-column scales are applied in the epilogue.
-template <int kDM, int WM, bool TRANS_B, bool SWIGLU, bool FP8>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+// NW wavefronts (4: one per SIMD; 8: two per SIMD, each with half the accumulators, so that one can issue MFMAs
+// while the other issues its reads and copies), WM of them along the rows.
+template <int kDM, int NW, int WM, bool TRANS_B, bool SWIGLU, bool FP8>
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW / 4, NW / 4)))
 void gmm_direct_kernel(const GmmArgs p) {
     constexpr int kStageK = FP8 ? 64 : kDK;               // k per stage: 64 bytes per row either way
     static_assert(!FP8 || TRANS_B, "fp8 operands are K-contiguous");
-    constexpr int WN = 4 / WM;                           // wavefronts along N
+    constexpr int WN = NW / WM;                          // wavefronts along N
     constexpr int TM = kDM / WM, TN = kDN / WN;          // wave tile
     constexpr int FM = TM / 32, FN = TN / 32;            // 32x32 accumulators per wavefront
     constexpr int NM = FM * FN;                          // MFMAs per k-step
     constexpr int NR = FM + FN;                          // operand reads per k-step (a B read = 2 transposing reads)
-    constexpr int CA = kDM / 64;                         // A copies (16 rows each) per wavefront per stage
-    constexpr int kLoads = CA + 4;                       // copies per wavefront per stage
+    constexpr int CA = kDM / (16 * NW);                  // A copies (16 rows each) per wavefront per stage
+    constexpr int CB = 16 / NW;                          // B copies (1 KiB of the 16 KiB each)
+    constexpr int kLoads = CA + CB;                      // copies per wavefront per stage
+    constexpr int kBlock = NW * 1024;                    // LDS bytes filled by one copy of every wavefront
     constexpr int kStageA = kDM * kDK * 2;
     constexpr int kStage = kStageA + kStageB;
     constexpr int kStages = kDM == 256 ? 4 : (kDM == 128 ? 5 : 6);
     constexpr int BNO = SWIGLU ? kDN / 2 : kDN;
     static_assert(kDM == 64 || kDM == 128 || kDM == 256, "tile rows");
-    static_assert(WM * WN == 4 && FM >= 1 && FN >= 2 && NR <= NM, "wave layout");
+    static_assert((NW == 4 || NW == 8) && WM * WN == NW && CA >= 1 && FM >= 1 && FN >= 2 && NR <= NM, "wave layout");
     static_assert((kStages - 1) * kLoads <= 63, "vmcnt is a 6-bit counter");
     extern __shared__ __attribute__((aligned(16))) char smem[];
     __shared__ int s_tile_start[kMaxGroups + 1];
@@ -110,7 +114,7 @@ void gmm_direct_kernel(const GmmArgs p) {
     const int kc_row = lane >> 2;
     const int kc_chunk = (lane & 3) ^ ((lane >> 4) & 3);      // logical chunk stored there
     // [k][n] image: a 1 KiB block is 2 k-rows of 512 B; lane l fills k-row l/32, physical chunk l%32
-    const int kn_k = 2 * wave + (lane >> 5);                  // k inside the stage, block i adds 8 i
+    const int kn_k = 2 * wave + (lane >> 5);                  // k inside the stage, block i adds 2 NW i
     const int kn_chunk = (lane & 31) ^ ((kn_k & 3) << 2);     // logical chunk (8 columns) stored there
 
     // ---- per-lane constants of the operand reads ----
@@ -125,7 +129,7 @@ void gmm_direct_kernel(const GmmArgs p) {
     // ---- state of the tile whose copies are being issued (set by open_tile) ----
     int e = 0, row0 = 0, rows_e = 0, n0 = 0;
     uint64_t a_base = 0, b_exp = 0;      // wave-uniform bases of the tile's rows of a and of the expert's weights
-    uint32_t a_off[CA], b_off[4];        // per-lane byte offsets of this wavefront's copies from those bases
+    uint32_t a_off[CA], b_off[CB];        // per-lane byte offsets of this wavefront's copies from those bases
 
     // tile column slot (0..255) -> column of b; slots past the end read the first column (never stored)
     auto b_col = [&](int slot) {
@@ -145,22 +149,22 @@ void gmm_direct_kernel(const GmmArgs p) {
         b_exp = to_scalar((uint64_t)(uintptr_t)p.b + (uint64_t)e * p.K * p.N * (FP8 ? 1 : 2));
 #pragma unroll
         for (int i = 0; i < CA; ++i) {
-            int r = (i * 4 + wave) * 16 + kc_row;
+            int r = (i * NW + wave) * 16 + kc_row;
             if (r >= rows_e) r = rows_e - 1;                   // clamp: loaded, never stored
             a_off[i] = (uint32_t)r * pitch + kc_chunk * 16;
         }
         if constexpr (TRANS_B) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) b_off[i] = (uint32_t)b_col((i * 4 + wave) * 16 + kc_row) * pitch + kc_chunk * 16;
+            for (int i = 0; i < CB; ++i) b_off[i] = (uint32_t)b_col((i * NW + wave) * 16 + kc_row) * pitch + kc_chunk * 16;
         } else {
-            // block i of this wavefront holds k-rows 8 i + kn_k of the stage
+            // block i of this wavefront holds k-rows 2 NW i + kn_k of the stage
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-                b_off[i] = (uint32_t)(i * 8 + kn_k) * (uint32_t)p.N * 2 + (uint32_t)b_col(kn_chunk * 8) * 2;
+            for (int i = 0; i < CB; ++i)
+                b_off[i] = (uint32_t)(i * 2 * NW + kn_k) * (uint32_t)p.N * 2 + (uint32_t)b_col(kn_chunk * 8) * 2;
         }
     };
 
-    // copy number c (0 .. kLoads-1) of this wavefront for stage s: first its CA blocks of A, then its 4 blocks of B
+    // copy number c (0 .. kLoads-1) of this wavefront for stage s: first its CA blocks of A, then its CB blocks of B
     auto issue_copy = [&](int s, auto c_tag) {
         constexpr int c = decltype(c_tag)::value;
 #ifdef DMOE_DEBUG_HOOKS
@@ -169,11 +173,11 @@ void gmm_direct_kernel(const GmmArgs p) {
 #endif
         const uint32_t lds = smem_addr + (s % kStages) * kStage + wave * 1024;
         if constexpr (c < CA) {
-            copy_g2lds_16<c * 4096>(a_off[c], a_base + (uint64_t)s * 64, lds);
+            copy_g2lds_16<c * kBlock>(a_off[c], a_base + (uint64_t)s * 64, lds);
         } else {
             constexpr int i = c - CA;
-            if constexpr (TRANS_B) copy_g2lds_16<kStageA + i * 4096>(b_off[i], b_exp + (uint64_t)s * 64, lds);
-            else copy_g2lds_16<kStageA + i * 4096>(b_off[i], b_exp + (uint64_t)s * kDK * p.N * 2, lds);
+            if constexpr (TRANS_B) copy_g2lds_16<kStageA + i * kBlock>(b_off[i], b_exp + (uint64_t)s * 64, lds);
+            else copy_g2lds_16<kStageA + i * kBlock>(b_off[i], b_exp + (uint64_t)s * kDK * p.N * 2, lds);
         }
     };
     const int pre = S < kStages ? S : kStages;      // stages whose copies are issued ahead of the tile's first MFMA
@@ -479,12 +483,12 @@ void gmm_direct_kernel(const GmmArgs p) {
     sched_finish(p.sched_slot);
 }
 
-template <int kDM, int WM, bool TRANS_B, bool SWIGLU, bool FP8>
+template <int kDM, int NW, int WM, bool TRANS_B, bool SWIGLU, bool FP8>
 static int launch_direct_one(const GmmArgs &args, hipStream_t stream) {
     constexpr int BNO = SWIGLU ? kDN / 2 : kDN;
     constexpr int kStages = kDM == 256 ? 4 : (kDM == 128 ? 5 : 6);
     const size_t lds = (size_t)kStages * (kDM * kDK * 2 + kStageB);
-    auto kern = gmm_direct_kernel<kDM, WM, TRANS_B, SWIGLU, FP8>;
+    auto kern = gmm_direct_kernel<kDM, NW, WM, TRANS_B, SWIGLU, FP8>;
     static unsigned long long configured = 0;   // devices on which the kernel's LDS size has been raised
     if (first_on_device(&configured))
         DMOE_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
@@ -497,30 +501,31 @@ static int launch_direct_one(const GmmArgs &args, hipStream_t stream) {
     GmmArgs launch_args = args;
     launch_args.sched_slot = next_sched_slot();
     launch_args.dbg = debug_mode();
-    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), lds, stream, launch_args);
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NW * 64), lds, stream, launch_args);
     DMOE_LAUNCH_CHECK("gmm_direct_kernel");
     return DMOE_OK;
 }
 
-template <int kDM, int WM>
+template <int kDM, int NW, int WM>
 static int launch_direct_tile(const GmmArgs &args, bool trans_b, bool swiglu, hipStream_t stream) {
-    if (trans_b) return swiglu ? launch_direct_one<kDM, WM, true, true, false>(args, stream) : launch_direct_one<kDM, WM, true, false, false>(args, stream);
-    return swiglu ? launch_direct_one<kDM, WM, false, true, false>(args, stream) : launch_direct_one<kDM, WM, false, false, false>(args, stream);
+    if (trans_b) return swiglu ? launch_direct_one<kDM, NW, WM, true, true, false>(args, stream) : launch_direct_one<kDM, NW, WM, true, false, false>(args, stream);
+    return swiglu ? launch_direct_one<kDM, NW, WM, false, true, false>(args, stream) : launch_direct_one<kDM, NW, WM, false, false, false>(args, stream);
 }
 
 // Preconditions (checked by the caller): bf16, K % 32 == 0, N % 8 == 0, K * N * 2 < 2^32.
-// tile_rows: 256, 128 or 64.
+// tile_rows: 256 (8 wavefronts), 128 or 64 (4 wavefronts); 260 = 256 rows on 4 wavefronts (comparison).
 int launch_direct_bf16(const GmmArgs &args, int tile_rows, bool trans_b, bool swiglu, hipStream_t stream) {
-    if (tile_rows == 64) return launch_direct_tile<64, 1>(args, trans_b, swiglu, stream);
-    if (tile_rows == 128) return launch_direct_tile<128, 2>(args, trans_b, swiglu, stream);
-    return launch_direct_tile<256, 2>(args, trans_b, swiglu, stream);
+    if (tile_rows == 64) return launch_direct_tile<64, 4, 1>(args, trans_b, swiglu, stream);
+    if (tile_rows == 128) return launch_direct_tile<128, 4, 2>(args, trans_b, swiglu, stream);
+    if (tile_rows == 260) return launch_direct_tile<256, 4, 2>(args, trans_b, swiglu, stream);   // 256 rows on 4 wavefronts
+    return launch_direct_tile<256, 8, 2>(args, trans_b, swiglu, stream);
 }
 
 // Preconditions: e4m3 operands, K-contiguous on both sides, K % 64 == 0, N % 8 == 0, K * N < 2^32.
 int launch_direct_fp8(const GmmArgs &args, int tile_rows, bool swiglu, hipStream_t stream) {
-    if (tile_rows == 64) return swiglu ? launch_direct_one<64, 1, true, true, true>(args, stream) : launch_direct_one<64, 1, true, false, true>(args, stream);
+    if (tile_rows == 64) return swiglu ? launch_direct_one<64, 4, 1, true, true, true>(args, stream) : launch_direct_one<64, 4, 1, true, false, true>(args, stream);
     // 256-row tiles would need 256 accumulator + 96 operand registers per lane plus addressing: they are cut in two
-    return swiglu ? launch_direct_one<128, 2, true, true, true>(args, stream) : launch_direct_one<128, 2, true, false, true>(args, stream);
+    return swiglu ? launch_direct_one<128, 4, 2, true, true, true>(args, stream) : launch_direct_one<128, 4, 2, true, false, true>(args, stream);
 }
 
 }  // namespace dmoe

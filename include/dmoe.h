@@ -159,7 +159,8 @@ int dmoe_gmm_workspace_bytes(int E, size_t *bytes);
  * kernel from rows per expert (default); 1 = register-staged 256x256 tile on 4
  * wavefronts; 2 = 64x256; 3 = 128x256; 4 = register-staged 256x256 tile on 8
  * wavefronts; 5, 6, 7 = the default kernels with tiles of 64, 128, 256 rows
- * whatever the rows per expert.  Process-wide, not thread-safe. */
+ * whatever the rows per expert; 8 = 256 rows on 4 instead of 8 wavefronts.
+ * Process-wide, not thread-safe. */
 int dmoe_gmm_tune(int variant);
 
 /* ---- fp8 (e4m3) path: no counterpart in the reference ---------------------

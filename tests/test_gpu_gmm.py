@@ -43,7 +43,7 @@ def test_reference_gemm_case():
     assert max_rel_err(y, ffn.gmm(x.cpu(), w1.cpu(), batch_sizes)) <= TOL_BF16
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, 8])
 @pytest.mark.parametrize("E,R,K,N", [(1, 300, 256, 256), (4, 1000, 128, 512), (8, 777, 320, 264), (3, 64, 72, 40),
                                      (5, 1500, 512, 768)])
 @pytest.mark.parametrize("trans_b", [False, True])
@@ -85,7 +85,7 @@ def test_gmm_single_expert_equals_matmul_and_zero_sizes():
     assert (guard[513:] == 5.0).all()
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, 8])
 @pytest.mark.parametrize("trans_b", [False, True])
 def test_gmm_swiglu(variant, trans_b):
     announce(test="gmm_swiglu", variant=variant, trans_b=trans_b)

@@ -13,9 +13,9 @@
 //       - B in the [K, N] layout is kept [k][256 n] (512 B rows): chunk ^ ((k & 3) << 2),
 //         read with ds_read_b64_tr_b16, which transposes 4 k x 16 n inside 16 lanes
 //         and hands every lane 4 consecutive k of its column - the MFMA B operand;
-//   * 4 wavefronts, one per SIMD; a wavefront owns 128x128 (256-row tile), 64x128 (128) or 64x64 (64) of
-//     the tile as 32x32 v_mfma_f32_32x32x16_bf16 accumulators; operands are double buffered in registers one
-//     k-step ahead; one workgroup barrier per stage.
+//   * 8 wavefronts (two per SIMD) on the 256-row tile, each with 128x64 of it; 4 wavefronts on the smaller tiles
+//     (64x128 of a 128-row tile, 64x64 of a 64-row tile); 32x32 v_mfma_f32_32x32x16_bf16 accumulators; operands are
+//     double buffered in registers one k-step ahead; one workgroup barrier per stage.
 #include "gmm_common.h"
 
 namespace dmoe {

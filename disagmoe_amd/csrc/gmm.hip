@@ -445,7 +445,7 @@ static int launch_by_rows(const GmmArgs &args, hipStream_t stream) {
     } else {
         // measured on the 8x22b shapes: with 256-row tiles the register-staged 8-wave kernel is ahead for the fused
         // gate-up projection, the direct kernel (128-row tiles at most) for the plain product
-        if (args.K % 64 == 0 && (long long)args.K * args.N < (1ll << 32) && !(SWIGLU && tile_rows == 256))
+        if (args.K % 64 == 0 && (long long)args.K * args.N < (1ll << 32))
             return launch_direct_fp8(args, tile_rows, SWIGLU, stream);
     }
     if (tile_rows == 64) return launch_one<64, 256, 1, 4, TRANS_B, SWIGLU, FP8>(args, stream);

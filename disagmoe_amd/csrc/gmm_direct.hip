@@ -203,7 +203,10 @@ void gmm_direct_kernel(const GmmArgs p) {
     }
 
     typedef typename std::conditional<FP8, i32x8, bf16x8>::type frag_t;
-    frag_t fa[FP8 ? 1 : 2][FM], fb[2][FN];
+    // fp8 on 8 wavefronts keeps a single register set for both operands: every fragment is re-read right behind its
+    // last MFMA of the stage, and the other wavefront of the SIMD covers the wait for the last of those reads
+    constexpr bool kOneSet = FP8 && NW == 8;
+    frag_t fa[FP8 ? 1 : 2][FM], fb[kOneSet ? 1 : 2][FN];
     // operand read number r (0 .. NR-1) of k-step ks of stage s into register set `slot`: first the FM A fragments,
     // then the FN B fragments
     auto load_frag = [&](int s, int ks, int slot, int r) {
@@ -316,7 +319,7 @@ void gmm_direct_kernel(const GmmArgs p) {
         // issue queues of all four wavefronts)
         auto run_stage = [&](int s, auto steady_tag, int ahead, bool next, bool deferred, auto odd_tag) {
             constexpr bool kSteady = decltype(steady_tag)::value;
-            constexpr int kCur = FP8 ? (decltype(odd_tag)::value ? 1 : 0) : 1;   // set used by the MFMAs after the hand-over
+            constexpr int kCur = FP8 ? (!kOneSet && decltype(odd_tag)::value ? 1 : 0) : 1;   // set used by the MFMAs after the hand-over
             constexpr int kFirst = FP8 ? kLoads : kLoads / 2;   // copies of stage s + kStages issued in this stage
             constexpr int kLate = kLoads - kFirst;              // ... and behind the MFMAs of k-step 0 of the next stage
             // bf16: copies go behind the MFMAs that have no operand read if those slots suffice
@@ -350,7 +353,11 @@ void gmm_direct_kernel(const GmmArgs p) {
                     // right behind their last MFMA of this stage; B fragments alternate between two sets.
                     mfma_one_fp8(kCur, t);
                     if (kSteady || next) {
-                        if (t < FN) load_frag(s + 1, 0, kCur ^ 1, FM + t);
+                        if constexpr (kOneSet) {
+                            if (t >= NM - FN) load_frag(s + 1, 0, 0, FM + t - (NM - FN));   // B fragment j, last used by MFMA t
+                        } else {
+                            if (t < FN) load_frag(s + 1, 0, kCur ^ 1, FM + t);
+                        }
                         if ((t % FN) == FN - 1) load_frag(s + 1, 0, 0, t / FN);
                     }
                 } else {
@@ -372,11 +379,11 @@ void gmm_direct_kernel(const GmmArgs p) {
             });
         };
         auto step = [&](int s, auto steady_tag, int ahead, bool next, bool deferred) {
-            if (FP8 && (s & 1)) run_stage(s, steady_tag, ahead, next, deferred, std::true_type{});
+            if (FP8 && !kOneSet && (s & 1)) run_stage(s, steady_tag, ahead, next, deferred, std::true_type{});
             else run_stage(s, steady_tag, ahead, next, deferred, std::false_type{});
         };
         int s = 0;
-        if constexpr (FP8) {
+        if constexpr (FP8 && !kOneSet) {
             // even and odd stages as one straight-line loop body: the accumulators stay where they are
             for (; s + 1 + kStages < S; s += 2) {
                 run_stage(s, std::true_type{}, 0, true, false, std::false_type{});
@@ -455,10 +462,14 @@ void gmm_direct_kernel(const GmmArgs p) {
         // fp8: one instance per wavefront number (the MFMA slots of its copies are compile-time constants)
         auto run_build = [&](auto guard_tag) {
             if constexpr (FP8) {
-                if (wave == 0) run_tile(guard_tag, std::integral_constant<int, 0>{});
-                else if (wave == 1) run_tile(guard_tag, std::integral_constant<int, 1>{});
-                else if (wave == 2) run_tile(guard_tag, std::integral_constant<int, 2>{});
-                else run_tile(guard_tag, std::integral_constant<int, 3>{});
+                if constexpr (NW == 8) {
+                    run_tile(guard_tag, std::integral_constant<int, 0>{});   // two wavefronts per SIMD: no staggering needed
+                } else {
+                    if (wave == 0) run_tile(guard_tag, std::integral_constant<int, 0>{});
+                    else if (wave == 1) run_tile(guard_tag, std::integral_constant<int, 1>{});
+                    else if (wave == 2) run_tile(guard_tag, std::integral_constant<int, 2>{});
+                    else run_tile(guard_tag, std::integral_constant<int, 3>{});
+                }
             } else {
                 run_tile(guard_tag, std::integral_constant<int, 0>{});
             }
@@ -524,7 +535,9 @@ int launch_direct_bf16(const GmmArgs &args, int tile_rows, bool trans_b, bool sw
 // Preconditions: e4m3 operands, K-contiguous on both sides, K % 64 == 0, N % 8 == 0, K * N < 2^32.
 int launch_direct_fp8(const GmmArgs &args, int tile_rows, bool swiglu, hipStream_t stream) {
     if (tile_rows == 64) return swiglu ? launch_direct_one<64, 4, 1, true, true, true>(args, stream) : launch_direct_one<64, 4, 1, true, false, true>(args, stream);
-    // 256-row tiles would need 256 accumulator + 96 operand registers per lane plus addressing: they are cut in two
+    // 256-row tiles: on 4 wavefronts they would need 256 accumulator + 96 operand registers per lane plus addressing;
+    // on 8 wavefronts a wavefront holds 128 + 48
+    if (tile_rows == 256) return swiglu ? launch_direct_one<256, 8, 2, true, true, true>(args, stream) : launch_direct_one<256, 8, 2, true, false, true>(args, stream);
     return swiglu ? launch_direct_one<128, 4, 2, true, true, true>(args, stream) : launch_direct_one<128, 4, 2, true, false, true>(args, stream);
 }
 

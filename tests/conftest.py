@@ -32,3 +32,12 @@ def pytest_collection_modifyitems(config, items):
 @pytest.fixture(scope="session")
 def golden_dir():
     return os.path.join(ROOT, "tests", "golden")
+
+
+@pytest.fixture(autouse=True)
+def _seeded():
+    # layers draw their random-init weights from torch's global generators: fix them so that a test sees the same
+    # weights in every run
+    import torch
+    torch.manual_seed(1234)
+    yield

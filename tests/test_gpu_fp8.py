@@ -46,8 +46,8 @@ def test_quantize_weight_matches_oracle():
     assert torch.equal(s.cpu(), s_ref) and torch.equal(q.cpu().view(torch.uint8), q_ref.view(torch.uint8))
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4])
-@pytest.mark.parametrize("E,R,K,N", [(1, 200, 256, 256), (4, 1000, 512, 520), (8, 700, 144, 264)])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7])
+@pytest.mark.parametrize("E,R,K,N", [(1, 200, 256, 256), (4, 1000, 512, 520), (8, 700, 144, 264), (3, 1300, 320, 384)])
 def test_gmm_fp8(variant, E, R, K, N):
     announce(test="gmm_fp8", variant=variant, E=E, R=R, K=K, N=N)
     gg.set_tile_variant(variant)
@@ -73,9 +73,19 @@ def test_gmm_fp8(variant, E, R, K, N):
         gg.set_tile_variant(0)
 
 
-def test_fp8_experts_forward():
-    announce(test="fp8_experts_forward")
-    E, d, I, R = 4, 512, 768, 600
+@pytest.mark.parametrize("variant,R", [(0, 600), (5, 600), (6, 600), (7, 600), (0, 1900)])
+def test_fp8_experts_forward(variant, R):
+    # variants 5, 6, 7: the 64-, 128- and 256-row tiles of the default kernels; 1900 rows pick the 256-row tile by themselves
+    announce(test="fp8_experts_forward", variant=variant, R=R)
+    gg.set_tile_variant(variant)
+    try:
+        _fp8_experts_forward(R)
+    finally:
+        gg.set_tile_variant(0)
+
+
+def _fp8_experts_forward(R):
+    E, d, I = 4, 512, 768
     g = torch.Generator().manual_seed(3)
     w13 = (torch.randn(E, d, 2 * I, generator=g) * 0.02).to(torch.bfloat16)
     w2 = (torch.randn(E, I, d, generator=g) * 0.02).to(torch.bfloat16)

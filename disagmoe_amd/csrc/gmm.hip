@@ -408,6 +408,7 @@ static int launch_one(const GmmArgs &args, hipStream_t stream) {
     long long grid = (long long)device_cus();
     if (m_tiles_max * n_tiles < grid) grid = m_tiles_max * n_tiles;
     if (grid < 1) grid = 1;
+    grid = (grid + kXcds - 1) / kXcds * kXcds;   // whole rows of XCDs: the tile order is XCD-aware only then
     GmmArgs launch_args = args;
     launch_args.sched_slot = next_sched_slot();
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NT), lds, stream, launch_args);
@@ -437,14 +438,15 @@ static int launch_by_rows(const GmmArgs &args, hipStream_t stream) {
         default: break;
     }
     int tile_rows = avg <= 64 ? 64 : (avg <= 160 ? 128 : 256);
+    // a tile size that would leave more than half of the CUs without a tile is halved (small problems: latency counts)
+    const long long n_tiles = ((SWIGLU ? args.N / 2 : args.N) + (SWIGLU ? 127 : 255)) / (SWIGLU ? 128 : 256);
+    while (tile_rows > 64 && (args.rows / tile_rows + (args.E + 1) / 2) * n_tiles * 2 < device_cus()) tile_rows /= 2;
     if (g_variant >= 5) tile_rows = g_variant == 5 ? 64 : (g_variant == 6 ? 128 : (g_variant == 7 ? 256 : 260));   // direct kernel, fixed tile rows (260: 256 rows on 4 wavefronts)
     if constexpr (!FP8) {
         // global -> LDS direct path: whole stages of 32 k, 32-bit offsets inside one expert's weights
         if (args.K % 32 == 0 && (long long)args.K * args.N * 2 < (1ll << 32))
             return launch_direct_bf16(args, tile_rows, TRANS_B, SWIGLU, stream);
     } else {
-        // measured on the 8x22b shapes: with 256-row tiles the register-staged 8-wave kernel is ahead for the fused
-        // gate-up projection, the direct kernel (128-row tiles at most) for the plain product
         if (args.K % 64 == 0 && (long long)args.K * args.N < (1ll << 32))
             return launch_direct_fp8(args, tile_rows, SWIGLU, stream);
     }

@@ -133,11 +133,16 @@ template <int BM>
 __device__ __forceinline__ TileCoord decode_tile(long long q, int G, long long total, int n_tiles, int E,
                                                  const int *s_tile_start, const int *s_row_start) {
     long long L = q;
-    const long long full_rounds = (G % kXcds == 0) ? total / G : 0;  // rounds in which the remap is a bijection
-    const long long round = q / G;
-    if (round < full_rounds) {
-        const int w = (int)(q - round * G);
-        L = round * G + (long long)(w % kXcds) * (G / kXcds) + (w / kXcds);
+    if (G % kXcds == 0) {
+        // a round holds cnt = min(G, items left) items; XCD x owns those with q % 8 == x, cnt / 8 of them plus one
+        // more on the first cnt % 8 XCDs, and they map onto consecutive tiles (a bijection for every cnt, so the
+        // last, partly filled round - the only round of a small problem - keeps its operand sharing too)
+        const long long base = (q / G) * G;
+        const long long left = total - base;
+        const int cnt = (int)(left < G ? left : G);
+        const int w = (int)(q - base), x = w % kXcds;
+        const int per = cnt / kXcds, extra = cnt % kXcds;
+        L = base + (long long)x * per + (x < extra ? x : extra) + (w / kXcds);
     }
     const int u = (int)(L / n_tiles);
     int lo = 0, hi = E;  // last e with s_tile_start[e] <= u

@@ -67,8 +67,11 @@ constexpr int kStageB = kDN * kDK * 2;     // 16 KiB of B per stage
 // v_mfma_f32_32x32x64_f8f6f4 k-step, and per-row / per-column scales are applied in the epilogue.
 // NW wavefronts (4: one per SIMD; 8: two per SIMD, each with half the accumulators, so that one can issue MFMAs
 // while the other issues its reads and copies), WM of them along the rows.
-template <int kDM, int NW, int WM, bool TRANS_B, bool SWIGLU, bool FP8>
-__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW / 4, NW / 4)))
+// NP = 0: every wavefront copies its share of a stage and computes.  NP = 2: wavefronts NW and NW + 1 only copy
+// (and draw the work items), the first NW only compute: a copy that waits for room in the memory pipeline then holds
+// up no MFMA, which is what small tiles on weights streamed from HBM need.
+template <int kDM, int NW, int WM, bool TRANS_B, bool SWIGLU, bool FP8, int NP = 0>
+__global__ __launch_bounds__((NW + NP) * 64) __attribute__((amdgpu_waves_per_eu((NW + NP + 3) / 4, (NW + NP + 3) / 4)))
 void gmm_direct_kernel(const GmmArgs p) {
     constexpr int kStageK = FP8 ? 64 : kDK;               // k per stage: 64 bytes per row either way
     static_assert(!FP8 || TRANS_B, "fp8 operands are K-contiguous");
@@ -77,16 +80,18 @@ void gmm_direct_kernel(const GmmArgs p) {
     constexpr int FM = TM / 32, FN = TN / 32;            // 32x32 accumulators per wavefront
     constexpr int NM = FM * FN;                          // MFMAs per k-step
     constexpr int NR = FM + FN;                          // operand reads per k-step (a B read = 2 transposing reads)
-    constexpr int CA = kDM / (16 * NW);                  // A copies (16 rows each) per wavefront per stage
-    constexpr int CB = 16 / NW;                          // B copies (1 KiB of the 16 KiB each)
-    constexpr int kLoads = CA + CB;                      // copies per wavefront per stage
-    constexpr int kBlock = NW * 1024;                    // LDS bytes filled by one copy of every wavefront
+    constexpr int NC = NP ? NP : NW;                     // wavefronts that copy
+    constexpr int CA = kDM / (16 * NC);                  // A copies (16 rows each) per copying wavefront per stage
+    constexpr int CB = 16 / NC;                          // B copies (1 KiB of the 16 KiB each)
+    constexpr int kLoads = CA + CB;                      // copies per copying wavefront per stage
+    constexpr int kBlock = NC * 1024;                    // LDS bytes filled by one copy of every copying wavefront
     constexpr int kStageA = kDM * kDK * 2;
     constexpr int kStage = kStageA + kStageB;
     constexpr int kStages = kDM == 256 ? 4 : (kDM == 128 ? 5 : 6);
     constexpr int BNO = SWIGLU ? kDN / 2 : kDN;
     static_assert(kDM == 64 || kDM == 128 || kDM == 256, "tile rows");
     static_assert((NW == 4 || NW == 8) && WM * WN == NW && CA >= 1 && FM >= 1 && FN >= 2 && NR <= NM, "wave layout");
+    static_assert(NP == 0 || (NP == 2 && NW == 4 && !FP8), "copying wavefronts: two, beside four computing ones");
     static_assert((kStages - 1) * kLoads <= 63, "vmcnt is a 6-bit counter");
     extern __shared__ __attribute__((aligned(16))) char smem[];
     __shared__ int s_tile_start[kMaxGroups + 1];
@@ -96,6 +101,7 @@ void gmm_direct_kernel(const GmmArgs p) {
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // kept in a scalar register: what derives from it stays wave-uniform
     const int wm = wave / WN, wn = wave % WN;
+    const int cw = NP ? wave - NW : wave;                      // number among the copying wavefronts (< 0: does not copy)
     const int E = p.E;
 
     build_work_list<kDM>(p, s_tile_start, s_row_start);
@@ -114,7 +120,7 @@ void gmm_direct_kernel(const GmmArgs p) {
     const int kc_row = lane >> 2;
     const int kc_chunk = (lane & 3) ^ ((lane >> 4) & 3);      // logical chunk stored there
     // [k][n] image: a 1 KiB block is 2 k-rows of 512 B; lane l fills k-row l/32, physical chunk l%32
-    const int kn_k = 2 * wave + (lane >> 5);                  // k inside the stage, block i adds 2 NW i
+    const int kn_k = 2 * cw + (lane >> 5);                    // k inside the stage, block i adds 2 NC i
     const int kn_chunk = (lane & 31) ^ ((kn_k & 3) << 2);     // logical chunk (8 columns) stored there
 
     // ---- per-lane constants of the operand reads ----
@@ -142,25 +148,28 @@ void gmm_direct_kernel(const GmmArgs p) {
         const int base = (SWIGLU && slot >= kDN / 2) ? n_out + nb : nb;
         return base + (rh < n_out - n0 ? rh : 0);
     };
-    auto open_tile = [&](long long q) {
+    auto locate_tile = [&](long long q) {
         const TileCoord tc = decode_tile<kDM>(q, G, total, n_tiles, E, s_tile_start, s_row_start);
         e = tc.e; row0 = tc.row0; rows_e = tc.rows_e; n0 = tc.nt * BNO;
+    };
+    auto open_tile = [&](long long q) {
+        locate_tile(q);
         a_base = to_scalar((uint64_t)(uintptr_t)p.a + (uint64_t)row0 * pitch);
         b_exp = to_scalar((uint64_t)(uintptr_t)p.b + (uint64_t)e * p.K * p.N * (FP8 ? 1 : 2));
 #pragma unroll
         for (int i = 0; i < CA; ++i) {
-            int r = (i * NW + wave) * 16 + kc_row;
+            int r = (i * NC + cw) * 16 + kc_row;
             if (r >= rows_e) r = rows_e - 1;                   // clamp: loaded, never stored
             a_off[i] = (uint32_t)r * pitch + kc_chunk * 16;
         }
         if constexpr (TRANS_B) {
 #pragma unroll
-            for (int i = 0; i < CB; ++i) b_off[i] = (uint32_t)b_col((i * NW + wave) * 16 + kc_row) * pitch + kc_chunk * 16;
+            for (int i = 0; i < CB; ++i) b_off[i] = (uint32_t)b_col((i * NC + cw) * 16 + kc_row) * pitch + kc_chunk * 16;
         } else {
-            // block i of this wavefront holds k-rows 2 NW i + kn_k of the stage
+            // block i of this wavefront holds k-rows 2 NC i + kn_k of the stage
 #pragma unroll
             for (int i = 0; i < CB; ++i)
-                b_off[i] = (uint32_t)(i * 2 * NW + kn_k) * (uint32_t)p.N * 2 + (uint32_t)b_col(kn_chunk * 8) * 2;
+                b_off[i] = (uint32_t)(i * 2 * NC + kn_k) * (uint32_t)p.N * 2 + (uint32_t)b_col(kn_chunk * 8) * 2;
         }
     };
 
@@ -171,7 +180,7 @@ void gmm_direct_kernel(const GmmArgs p) {
         // timing experiments (wrong results): 1 = no copies after the prologue, 2 = no A copies, 3 = no B copies
         if (s >= kStages && (p.dbg == 1 || (p.dbg == 2 && c < CA) || (p.dbg == 3 && c >= CA))) return;
 #endif
-        const uint32_t lds = smem_addr + (s % kStages) * kStage + wave * 1024;
+        const uint32_t lds = smem_addr + (s % kStages) * kStage + cw * 1024;
         if constexpr (c < CA) {
             copy_g2lds_16<c * kBlock>(a_off[c], a_base + (uint64_t)s * 64, lds);
         } else {
@@ -252,7 +261,8 @@ void gmm_direct_kernel(const GmmArgs p) {
 
     // ---- first work item ----
     unsigned int draw = 0;
-    if (tid == 0) {
+    const bool drawer = tid == (NP ? NW * 64 : 0);
+    if (drawer) {
         draw = sched_draw(p.sched_slot, streams);
         s_item = sched_item(draw, streams);
         draw = sched_draw(p.sched_slot, streams);   // always one draw ahead: its round trip hides behind a tile
@@ -260,8 +270,38 @@ void gmm_direct_kernel(const GmmArgs p) {
     __syncthreads();
     long long q = s_item;
     if (q < total) {
-        open_tile(q);
-        issue_prologue();
+        if (NP == 0 || cw >= 0) {
+            open_tile(q);
+            issue_prologue();
+        } else {
+            locate_tile(q);
+        }
+    }
+
+    if constexpr (NP > 0) {
+        if (cw >= 0) {
+            // ---- a copying wavefront: the same barriers as the computing ones, tile by tile ----
+            while (q < total) {
+                wait_ahead(pre - 1);
+                __syncthreads();                   // stage 0 has landed
+                for (int s = 0; s + 1 < S; ++s) {
+                    const int left = S - 1 - s;    // stages after s; s + 1 has to land, the ones behind it may be in flight
+                    wait_ahead(left - 1 < kStages - 2 ? left - 1 : kStages - 2);
+                    __syncthreads();               // hand-over: stage s + 1 is there, stage s has been read
+                    if (s + kStages < S) static_for<0, kLoads>([&](auto c) { issue_copy(s + kStages, c); });
+                }
+                if (drawer) s_item = sched_item(draw, streams);
+                __syncthreads();                   // the last stage has been read: all of the LDS may be refilled
+                q = s_item;
+                if (q < total) {
+                    if (drawer) draw = sched_draw(p.sched_slot, streams);
+                    open_tile(q);
+                    issue_prologue();
+                }
+            }
+            sched_finish(p.sched_slot);
+            return;
+        }
     }
 
     while (q < total) {
@@ -298,7 +338,7 @@ void gmm_direct_kernel(const GmmArgs p) {
 
         // stage 0 of this tile has landed (its other prologue stages, and stores of the previous tile's
         // epilogue that were issued after them, may still be in flight: waiting for fewer is only stricter)
-        wait_ahead(pre - 1);
+        if constexpr (NP == 0) wait_ahead(pre - 1);
         __syncthreads();
 #pragma unroll
         for (int r = 0; r < NR; ++r) load_frag(0, 0, 0, r);
@@ -329,7 +369,7 @@ void gmm_direct_kernel(const GmmArgs p) {
                     constexpr int t = decltype(t_tag)::value;
                     mfma_one(0, t);
                     if (t < NR) load_frag(s, 1, 1, t);
-                    if (deferred) {
+                    if (NP == 0 && deferred) {
                         static_for<copy_slot(t, kLate, kSlot0, NM), copy_slot(t + 1, kLate, kSlot0, NM)>(
                             [&](auto c) { issue_copy(s - 1 + kStages, std::integral_constant<int, kFirst + decltype(c)::value>{}); });
                     }
@@ -341,7 +381,8 @@ void gmm_direct_kernel(const GmmArgs p) {
                 if (kSteady && p.dbg == 13) {}   // timing experiment (wrong results): no wait for the copies
                 else
 #endif
-                if constexpr (kSteady) DMOE_WAIT_VMCNT((kStages - 2) * kLoads);
+                if constexpr (NP > 0) {}   // the copying wavefronts wait for the data
+                else if constexpr (kSteady) DMOE_WAIT_VMCNT((kStages - 2) * kLoads);
                 else wait_ahead(ahead);
                 __syncthreads();
                 __builtin_amdgcn_sched_barrier(0);
@@ -364,7 +405,7 @@ void gmm_direct_kernel(const GmmArgs p) {
                     mfma_one(kCur, t);
                     if ((kSteady || next) && t < NR) load_frag(s + 1, 0, kCur ^ 1, t);
                 }
-                if constexpr (kSteady) {
+                if constexpr (kSteady && NP == 0) {
                     if constexpr (FP8) {
                         static_for<0, kFirst>([&](auto c) {
                             if constexpr (copy_slot_of(decltype(c)::value, kFirst, NM, decltype(phase_tag)::value) == t)
@@ -397,6 +438,11 @@ void gmm_direct_kernel(const GmmArgs p) {
             const int left = S - 1 - s;                           // stages after this one
             step(s, std::false_type{}, left - 1 < kStages - 2 ? left - 1 : kStages - 2, left > 0,
                  !FP8 && s > 0 && s + kStages == S);
+        }
+
+        if constexpr (NP > 0) {
+            __syncthreads();   // every wavefront has read its last fragments: the copying wavefronts may refill the LDS
+            q = s_item;        // the next work item, written by them before the barrier
         }
 
         auto epilogue = [&]() {
@@ -479,27 +525,28 @@ void gmm_direct_kernel(const GmmArgs p) {
 
         auto next_item = [&]() {
             // ---- next work item and its first copies ----
-            if (tid == 0) s_item = sched_item(draw, streams);
+            if (drawer) s_item = sched_item(draw, streams);
             __syncthreads();   // also: the last stage has been read by everyone, LDS may be refilled
             q = s_item;
             if (q < total) {
-                if (tid == 0) draw = sched_draw(p.sched_slot, streams);
+                if (drawer) draw = sched_draw(p.sched_slot, streams);
                 open_tile(q);
                 issue_prologue();
             }
         };
         // stores first: they are then older than the next tile's copies and never hold up a vmcnt wait of its pipeline
-        next_item();
+        if constexpr (NP == 0) next_item();
+        else if (q < total) locate_tile(q);
     }
     sched_finish(p.sched_slot);
 }
 
-template <int kDM, int NW, int WM, bool TRANS_B, bool SWIGLU, bool FP8>
+template <int kDM, int NW, int WM, bool TRANS_B, bool SWIGLU, bool FP8, int NP = 0>
 static int launch_direct_one(const GmmArgs &args, hipStream_t stream) {
     constexpr int BNO = SWIGLU ? kDN / 2 : kDN;
     constexpr int kStages = kDM == 256 ? 4 : (kDM == 128 ? 5 : 6);
     const size_t lds = (size_t)kStages * (kDM * kDK * 2 + kStageB);
-    auto kern = gmm_direct_kernel<kDM, NW, WM, TRANS_B, SWIGLU, FP8>;
+    auto kern = gmm_direct_kernel<kDM, NW, WM, TRANS_B, SWIGLU, FP8, NP>;
     static unsigned long long configured = 0;   // devices on which the kernel's LDS size has been raised
     if (first_on_device(&configured))
         DMOE_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
@@ -509,24 +556,26 @@ static int launch_direct_one(const GmmArgs &args, hipStream_t stream) {
     long long grid = (long long)device_cus();
     if (m_tiles_max * n_tiles < grid) grid = m_tiles_max * n_tiles;
     if (grid < 1) grid = 1;
+    grid = (grid + kXcds - 1) / kXcds * kXcds;   // whole rows of XCDs: the tile order is XCD-aware only then
     GmmArgs launch_args = args;
     launch_args.sched_slot = next_sched_slot();
     launch_args.dbg = debug_mode();
-    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NW * 64), lds, stream, launch_args);
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3((NW + NP) * 64), lds, stream, launch_args);
     DMOE_LAUNCH_CHECK("gmm_direct_kernel");
     return DMOE_OK;
 }
 
-template <int kDM, int NW, int WM>
+template <int kDM, int NW, int WM, int NP = 0>
 static int launch_direct_tile(const GmmArgs &args, bool trans_b, bool swiglu, hipStream_t stream) {
-    if (trans_b) return swiglu ? launch_direct_one<kDM, NW, WM, true, true, false>(args, stream) : launch_direct_one<kDM, NW, WM, true, false, false>(args, stream);
-    return swiglu ? launch_direct_one<kDM, NW, WM, false, true, false>(args, stream) : launch_direct_one<kDM, NW, WM, false, false, false>(args, stream);
+    if (trans_b) return swiglu ? launch_direct_one<kDM, NW, WM, true, true, false, NP>(args, stream) : launch_direct_one<kDM, NW, WM, true, false, false, NP>(args, stream);
+    return swiglu ? launch_direct_one<kDM, NW, WM, false, true, false, NP>(args, stream) : launch_direct_one<kDM, NW, WM, false, false, false, NP>(args, stream);
 }
 
 // Preconditions (checked by the caller): bf16, K % 32 == 0, N % 8 == 0, K * N * 2 < 2^32.
-// tile_rows: 256 (8 wavefronts), 128 or 64 (4 wavefronts); 260 = 256 rows on 4 wavefronts (comparison).
+// tile_rows: 256 (8 wavefronts), 128 (4 wavefronts) or 64 (4 computing + 2 copying wavefronts); 260 = 256 rows on 4
+// wavefronts (comparison).
 int launch_direct_bf16(const GmmArgs &args, int tile_rows, bool trans_b, bool swiglu, hipStream_t stream) {
-    if (tile_rows == 64) return launch_direct_tile<64, 4, 1>(args, trans_b, swiglu, stream);
+    if (tile_rows == 64) return launch_direct_tile<64, 4, 1, 2>(args, trans_b, swiglu, stream);   // 4 + 2 copying wavefronts
     if (tile_rows == 128) return launch_direct_tile<128, 4, 2>(args, trans_b, swiglu, stream);
     if (tile_rows == 260) return launch_direct_tile<256, 4, 2>(args, trans_b, swiglu, stream);   // 256 rows on 4 wavefronts
     return launch_direct_tile<256, 8, 2>(args, trans_b, swiglu, stream);

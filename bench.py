@@ -29,6 +29,17 @@ PEAK_FP8_TFLOPS = 5000.0
 MEASURED_TRAFFIC = {"C2": 6.36e9}
 
 
+def _tile_rows(w) -> int:
+    """Tile rows the gate-up launch gets: mirrors launch_by_rows (csrc/gmm.hip)."""
+    avg = w.R // w.E
+    tile = 64 if avg <= 64 else (128 if avg <= 160 else 256)
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    n_tiles = (w.I + 127) // 128
+    while tile > 64 and (w.R // tile + (w.E + 1) // 2) * n_tiles * 2 < cus:
+        tile //= 2
+    return tile
+
+
 def _event_ms(fn, iters: int, warmup: int = 2):
     """Average duration of ``fn`` in ms, HIP events on the current stream (the one
     the kernels are launched on)."""
@@ -168,11 +179,9 @@ def main() -> int:
         q_ms, _ = _event_ms(lambda: gg.quantize_rows(permuted), it)
         stages["quant_rows"] = {"ms": q_ms}
         peak = PEAK_FP8_TFLOPS
-        avg = w.R // w.E
-        tile = 64 if avg <= 64 else (128 if avg <= 160 else 256)
-        # mirrors the dispatch of launch_by_rows (csrc/gmm.hip): the fused fp8 gate-up projection on 256-row tiles
-        # runs on the register-staged kernel, every other case on the global-to-LDS kernel
-        kernel = ("dmoe::gmm_kernel<256, 256, .., swiglu, fp8>" if tile == 256 or w.d % 64 or w.d < 448
+        tile = _tile_rows(w)
+        # mirrors the dispatch of launch_by_rows (csrc/gmm.hip): the global-to-LDS kernel takes whole 64-k stages
+        kernel = (f"dmoe::gmm_kernel<{tile}, 256, .., swiglu, fp8>" if w.d % 64
                   else f"dmoe::gmm_direct_kernel<{tile}, .., swiglu, fp8>") + " (gate-up projection with fused SiLU*mul)"
     else:
         h = gg.gmm_swiglu(permuted, layer.w13_weight, batch_sizes)
@@ -180,9 +189,8 @@ def main() -> int:
         y_buf = torch.empty((w.R, w.d), dtype=torch.bfloat16, device=dev)
         down_ms, _ = _event_ms(lambda: gg.gmm(h, layer.w2_weight, batch_sizes, c=y_buf), it)
         peak = PEAK_BF16_TFLOPS
-        avg = w.R // w.E
-        tile = 64 if avg <= 64 else (128 if avg <= 160 else 256)
-        direct = w.d % 32 == 0 and w.d >= 224
+        tile = _tile_rows(w)
+        direct = w.d % 32 == 0
         kernel = (f"dmoe::gmm_direct_kernel<{tile}, .., [K,N] weights, swiglu, bf16>" if direct
                   else f"dmoe::gmm_kernel<{tile}, 256, .., swiglu, bf16>") + " (gate-up projection with fused SiLU*mul)"
     up_flops = 2.0 * w.R * w.d * 2 * w.I

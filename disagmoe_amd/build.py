@@ -14,7 +14,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_PATH = os.path.join(HERE, "libdmoe_hip.so")
-SOURCES = ["route.hip", "topk.hip", "rows.hip", "gmm.hip", "gmm_direct.hip"]
+SOURCES = ["route.hip", "topk.hip", "rows.hip", "meta.hip", "gmm.hip", "gmm_direct.hip"]
 ARCH = "gfx950"
 
 FLAGS = [

@@ -15,6 +15,7 @@ import torch
 
 from . import _lib
 from .ops import memory
+from .ops.metadata import Metadata
 
 
 def expert_layer_forward(experts: torch.nn.Module, x: torch.Tensor, topk_ids: torch.Tensor,
@@ -33,3 +34,35 @@ def expert_layer_forward(experts: torch.nn.Module, x: torch.Tensor, topk_ids: to
         stages.update(mappings=mappings, batch_sizes=batch_sizes, offsets=offsets, permuted=permuted,
                       expert_out=expert_out)
     return out
+
+
+def process_batch_expert(executor, meta: Metadata, input_tensor: torch.Tensor,
+                         inner_exp_rank=None, top_k: int = 1):
+    """The expert worker's step on a batch that arrives sorted by expert id
+    (disagmoe/frontend/engine.py:683-739): batch sizes of the local experts from the
+    bookkeeping, the FFN, then the rows go back to prefill-then-decode order, scaled by
+    their top-k weights on the way (one kernel: the scale is an argument of the permute).
+    ``executor`` is an ``ExpertsExecutor``; returns ``(output, meta)`` like the reference.
+
+    A row is scaled by its own weight.  The reference builds the weight tensor from the lists
+    after ``sort_by_prefill_order`` has reordered them (engine.py:715, then :726) and multiplies
+    rows that are still in expert order (:732), which pairs rows with other rows' weights
+    whenever the return mapping is not the identity; that is not reproduced."""
+    num_tokens = meta.num_tokens()
+    dev = input_tensor.device
+    num_experts = executor.model_config.num_experts
+    sizes = meta.get_expert_batch_sizes(num_experts)
+    if inner_exp_rank is not None:
+        sizes = [sizes[i] for i in inner_exp_rank]
+    batch_sizes = torch.tensor(sizes, dtype=torch.int64).to(dev, non_blocking=True)
+    output = executor.execute(meta.layer_id, num_tokens, input_tensor, batch_sizes)
+    # the weights travel with the rows: read them before the lists are reordered
+    weights = None
+    if top_k > 1:
+        weights = torch.tensor(meta.topk_weights, dtype=output.dtype).to(dev, non_blocking=True)
+    new_mappings = meta.sort_by_prefill_order()
+    mappings = torch.tensor(new_mappings, dtype=torch.int64).to(dev, non_blocking=True)
+    output = memory.permute_tokens_cuda(output, mappings, row_scale=weights)
+    meta.update_exp_ids([], [])
+    meta.step_layer()
+    return output, meta

@@ -93,6 +93,31 @@ int dmoe_route(const void *ids, int ids_type, int64_t R, int E, int order,
 int dmoe_topk_softmax(const void *logits, int logits_dtype, int64_t n, int E, int k, int renormalize,
                       float *weights, void *ids, int ids_type, void *stream);
 
+/* ---- per-row bookkeeping (host arrays, no device work) --------------------
+ * The integer lists that travel with a batch on the expert worker: request
+ * id, expert id, attention DP rank, initial prefill length per row.
+ *
+ * dmoe_sort_by_prefill_order replaces Metadata::sort_by_prefill_order
+ * (csrc/include/datatypes.hpp:411-433): rows ranked by DP rank, then prefill
+ * rows (init_prefill_len != -1) before decode rows, prefill rows by request
+ * id; mapping[rank[i]] = i is the return permute of
+ * disagmoe/frontend/engine.py:715,734.  The reference leaves rows that compare
+ * equal to a non-stable sort; here they keep their order.
+ *
+ * dmoe_move_row_infos replaces Metadata::permute_token_infos (:377-409) for one
+ * list: out[mapping[i]] = values[i], elements of 4 or 8 bytes, out != values.
+ *
+ * dmoe_expert_batch_sizes replaces Metadata::get_expert_batch_sizes and the
+ * selection of the local experts in get_expert_batch_sizes_cuda (:228-247):
+ * histogram of exp_ids over n_expert experts; with inner_exp_rank (m entries)
+ * batches[i] = hist[inner_exp_rank[i]], without it batches[e] = hist[e].  Any
+ * number of experts (the reference's stack buffer holds 8). */
+int dmoe_sort_by_prefill_order(const int32_t *req_ids, const int32_t *attn_dp_ranks,
+                               const int32_t *init_prefill_lens, int64_t n, int64_t *mapping);
+int dmoe_move_row_infos(const void *values, int elem_bytes, const int64_t *mapping, int64_t n, void *out);
+int dmoe_expert_batch_sizes(const int32_t *exp_ids, int64_t n, int n_expert, const int32_t *inner_exp_rank, int m,
+                            int64_t *batches);
+
 /* ---- row movement -------------------------------------------------------
  * dmoe_permute replaces permute_tokens_cuda(tokens, mappings, stream)
  * (csrc/include/permute.h:8, csrc/cuda_ops/permute.cu:86-112, bound at

@@ -88,3 +88,52 @@ def test_full_size_layer(name, rows_per_expert):
     ref_out = ffn.combine(y.cpu(), m_ref, gates)
     assert max_rel_err(out, ref_out) <= 2 ** -7
     assert torch.isfinite(out.float()).all()
+
+
+@pytest.mark.parametrize("top_k", [1, 2])
+def test_process_batch_expert(top_k):
+    # the expert worker's step on an expert-sorted batch (engine.py:683-739): FFN, scale by the row's top-k weight,
+    # rows back to prefill-then-decode order; lists of the bookkeeping moved along
+    from disagmoe_amd.config import ModelConfig
+    from disagmoe_amd.executor import ExpertsExecutor
+    from disagmoe_amd.expert_layer import process_batch_expert
+    from disagmoe_amd.ops.metadata import Metadata
+    announce(test="process_batch_expert", top_k=top_k)
+    E, d, I, R = 4, 512, 768, 300
+    cfg = ModelConfig(hidden_size=d, num_layers=1, num_heads=8, num_kv_heads=8, num_experts=E, intermediate_size=I,
+                      layer_ids=[0], top_k=top_k)
+    ex = ExpertsExecutor(cfg, init_std=0.02)
+    g = torch.Generator().manual_seed(5)
+    exp_ids = torch.sort(torch.randint(0, E, (R,), generator=g)).values.tolist()          # arrives sorted by expert
+    req_ids = torch.randperm(R, generator=g).tolist()
+    lens = torch.where(torch.rand(R, generator=g) < 0.5, -1, 8).tolist()
+    dp = torch.randint(0, 2, (R,), generator=g).tolist()
+    weights = torch.rand(R, generator=g).tolist() if top_k > 1 else []
+    x = torch.randn(R, d, generator=g).to(torch.bfloat16)
+    meta = Metadata(shape=[R, d], layer_id=0, req_ids=list(req_ids), exp_ids=list(exp_ids), attn_dp_ranks=list(dp),
+                    init_prefill_lens=list(lens), topk_weights=list(weights))
+    out, new_meta = process_batch_expert(ex, meta, x.to(dev()), top_k=top_k)
+
+    op = ex.operators[0]
+    sizes = routing.expert_batch_sizes(exp_ids, E).tolist()
+    y = ffn.moe_experts_forward(x, op.w13_weight.cpu(), op.w2_weight.cpu(), sizes)
+    if top_k > 1:
+        y = (y.float() * torch.tensor(weights).to(torch.bfloat16).float().view(-1, 1)).to(torch.bfloat16)
+    mapping = routing.sort_by_prefill_order(req_ids, dp, lens)
+    ref = torch.empty_like(y)
+    ref[torch.tensor(mapping)] = y
+    assert out.shape == (R, d)
+    assert max_rel_err(out, ref) <= TOL_BF16, max_rel_err(out, ref)
+    # bookkeeping: lists in the new order, expert ids dropped, layer stepped
+    assert new_meta.req_ids == routing.apply_row_mapping(req_ids, mapping)
+    assert new_meta.init_prefill_lens == routing.apply_row_mapping(lens, mapping)
+    assert new_meta.exp_ids == [] and new_meta.layer_id == 1
+    order = [(a, p == -1) for a, p in zip(new_meta.attn_dp_ranks, new_meta.init_prefill_lens)]
+    assert order == sorted(order)
+    # the data movement alone is exact: same FFN output scaled and moved by torch
+    y_dev = op.forward(R, x.to(dev()), torch.tensor(sizes, device=dev()))
+    if top_k > 1:
+        y_dev = y_dev * torch.tensor(weights, dtype=torch.bfloat16, device=dev()).view(-1, 1)
+    moved = torch.empty_like(y_dev)
+    moved[torch.tensor(mapping, device=dev())] = y_dev
+    assert torch.equal(out, moved)

@@ -31,6 +31,7 @@ MEASURED_TRAFFIC = {"C2": 6.36e9}
 
 def _tile_rows(w) -> int:
     """Tile rows the gate-up launch gets: mirrors launch_by_rows (csrc/gmm.hip)."""
+    import torch
     avg = w.R // w.E
     tile = 64 if avg <= 64 else (128 if avg <= 160 else 256)
     cus = torch.cuda.get_device_properties(0).multi_processor_count

@@ -145,3 +145,23 @@ def test_serial_experts_and_executor():
     assert max_rel_err(serial.forward(R, x, sizes), ref) <= TOL_BF16
     cfg.enable_grouped_gemm = False
     assert isinstance(ExpertsExecutor(cfg, init_std=0.02).operators[0], MoEExpertsSerial)
+
+
+@pytest.mark.parametrize("trans_b", [False, True])
+def test_gmm_expert_count_limit(trans_b):
+    # the tile tables of E + 1 entries live in LDS: up to 1024 experts per call, most of them empty here
+    announce(test="gmm_max_experts", trans_b=trans_b)
+    from disagmoe_amd._lib import DmoeError
+    E, R, K, N = 1024, 700, 128, 256
+    g = torch.Generator().manual_seed(3)
+    sizes = torch.zeros(E, dtype=torch.int64)
+    picks = torch.randperm(E, generator=g)[:40]
+    sizes[picks] = torch.randint(1, 30, (40,), generator=g)
+    sizes[picks[0]] += R - int(sizes.sum())
+    assert int(sizes.sum()) == R and int(sizes.min()) == 0
+    a = _rand((R, K), 21)
+    b = _rand((E, N, K) if trans_b else (E, K, N), 22, std=0.05)
+    out = gg.gmm(a.to(dev()), b.to(dev()), sizes.to(dev()), trans_b=trans_b)
+    assert max_rel_err(out, ffn.gmm(a, b, sizes, trans_b=trans_b)) <= TOL_BF16
+    with pytest.raises(DmoeError):
+        gg.gmm(a.to(dev()), _rand((1025, K, 8), 23).to(dev()), torch.zeros(1025, dtype=torch.int64), trans_b=False)

@@ -99,3 +99,14 @@ def test_merge_of_several_batches():
     flat = torch.tensor([v for b in batches for v in b], dtype=torch.int32, device=dev())
     m, bs, _ = memory.route_tokens(flat, 8)
     assert m.cpu().tolist() == m_ref and bs.cpu().tolist() == cnt_ref
+
+
+def test_expert_count_limits():
+    # the routing tables of E entries live in LDS: up to 4096 experts, more is refused
+    announce(test="route_max_experts")
+    from disagmoe_amd._lib import DmoeError
+    g = torch.Generator().manual_seed(11)
+    _check(torch.randint(0, 4096, (10000,), generator=g), 4096)
+    _check(torch.randint(4000, 4096, (300,), generator=g), 4096)      # one chunk, nearly all experts empty
+    with pytest.raises(DmoeError):
+        memory.route_tokens(torch.zeros(8, dtype=torch.int64, device=dev()), 4097)

@@ -165,3 +165,25 @@ def test_gmm_expert_count_limit(trans_b):
     assert max_rel_err(out, ffn.gmm(a, b, sizes, trans_b=trans_b)) <= TOL_BF16
     with pytest.raises(DmoeError):
         gg.gmm(a.to(dev()), _rand((1025, K, 8), 23).to(dev()), torch.zeros(1025, dtype=torch.int64), trans_b=False)
+
+
+@pytest.mark.parametrize("trans_b", [False, True])
+def test_gmm_weights_beyond_32bit_offsets(trans_b):
+    # one expert's weights of 2^32 bytes and more leave the kernel with 32-bit offsets inside an expert; columns at
+    # both ends and around the 2^31 / 2^32 byte marks are compared with the oracle
+    announce(test="gmm_4gib_expert", trans_b=trans_b)
+    E, R, K, N = 2, 96, 16384, 131072 + 256
+    g = torch.Generator(device=dev()).manual_seed(9)
+    b = torch.empty((E, N, K) if trans_b else (E, K, N), dtype=torch.bfloat16, device=dev())
+    for e in range(E):
+        b[e].copy_(torch.randn(b.shape[1:], device=dev(), generator=g, dtype=torch.float32).mul_(0.02))
+    a = _rand((R, K), 31)
+    sizes = torch.tensor([40, 56])
+    out = gg.gmm(a.to(dev()), b, sizes, trans_b=trans_b)
+    assert out.shape == (R, N)
+    cols = torch.cat([torch.arange(0, 64), torch.arange(65536 - 32, 65536 + 32), torch.arange(131072 - 32, 131072 + 32),
+                      torch.arange(N - 64, N)])
+    b_cols = (b[:, cols, :].transpose(1, 2) if trans_b else b[:, :, cols]).contiguous().cpu()
+    ref = ffn.gmm(a, b_cols, sizes)
+    assert max_rel_err(out[:, cols.to(dev())], ref) <= TOL_BF16
+    assert torch.isfinite(out.float()).all()

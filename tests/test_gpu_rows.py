@@ -151,3 +151,25 @@ def test_full_size_permute_and_combine(name):
         assert torch.equal(p.cpu(), rows.permute_tokens(x.cpu(), m.cpu()))
         out = memory.combine_tokens(p, m, gates.to(dev()))
         assert max_rel_err(out, ffn.combine(p.cpu(), m.cpu(), gates)) <= 2 ** -7
+
+
+def test_row_buffers_beyond_4gib():
+    # 640k routed rows of 8 KiB: byte offsets pass 2^32 in the source and the destination of every row kernel
+    T, d, k, E = 320000, 4096, 2, 8
+    announce(test="rows_beyond_4gib", T=T, d=d, k=k)
+    g = torch.Generator(device=dev()).manual_seed(4)
+    x = torch.randn(T, d, device=dev(), generator=g, dtype=torch.float32).to(torch.bfloat16)
+    ids = torch.randint(0, E, (T, k), device=dev(), generator=g, dtype=torch.int32)
+    m, bs, off = memory.route_tokens(ids, E)
+    assert int(bs.sum()) == T * k
+    p = memory.permute_tokens_cuda(x, m)
+    assert p.numel() * 2 > 2 ** 32
+    # every routed row t sits at mappings[t]; checked in slabs to bound the checker's memory
+    for lo in range(0, T, 80000):
+        rows_t = torch.arange(lo * k, (lo + 80000) * k, device=dev())
+        assert torch.equal(p[m[rows_t]], x[lo:lo + 80000].repeat_interleave(k, dim=0))
+    back = memory.gather_rows(p, m.view(T, k)[:, 1].contiguous())
+    assert torch.equal(back, x)
+    first = torch.zeros(T, k, device=dev())
+    first[:, 0] = 1
+    assert torch.equal(memory.combine_tokens(p, m, first), x)

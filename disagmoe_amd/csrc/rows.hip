@@ -128,7 +128,7 @@ template <bool kHalf>
 __device__ __forceinline__ uint16_t f32_to_elem(float f) { return kHalf ? f32_to_half_bits(f) : f32_to_bf16(f); }
 
 // out[i] = sum_j w[i,j] * y[map[i*k+j]]; one wavefront per (token i, segment).
-template <typename MapT, bool kHalf, int kMode>
+template <typename MapT, bool kHalf, int kMode, bool kStreamed>
 __global__ __launch_bounds__(kBlock) void combine_kernel(const u32x4 *__restrict__ y, const MapT *__restrict__ map,
                                                         const float *__restrict__ w, u32x4 *__restrict__ out,
                                                         int64_t T, int k, int64_t R, int vecs, int nseg) {
@@ -156,7 +156,8 @@ __global__ __launch_bounds__(kBlock) void combine_kernel(const u32x4 *__restrict
         for (int u = 0; u < kVecs; ++u) {
             const int v = v0 + u * kWave;
             buf[u] = u32x4{0, 0, 0, 0};
-            if (v < vecs) buf[u] = src[v];
+            // every row of y is read once; when y is larger than the last-level cache the loads say so
+            if (v < vecs) buf[u] = kStreamed ? __builtin_nontemporal_load(src + v) : src[v];
         }
 #pragma unroll
         for (int u = 0; u < kVecs; ++u) {
@@ -364,9 +365,17 @@ extern "C" int dmoe_combine(const void *y, const void *mappings, int map_type, c
     const int64_t nblk = blocks_for(T * nseg);
     DMOE_REQUIRE(nblk < (1ll << 31), DMOE_ERR_SHAPE, "dmoe_combine: too many rows");
     hipStream_t s = (hipStream_t)stream;
+    // measured: non-temporal loads of y are 20 % faster on 403 MB of rows and 8 % slower on 67 and 201 MB, which the
+    // 256 MB Infinity Cache can still hold between the GEMM that wrote them and this kernel
+    const bool streamed = R * (int64_t)vecs * 16 > (256ll << 20);
+#define DMOE_COMBINE_LAUNCH_ONE(MAPT, HALF, MODE, STREAMED)                                                           \
+    hipLaunchKernelGGL((combine_kernel<MAPT, HALF, MODE, STREAMED>), dim3((unsigned)nblk), dim3(kBlock), 0, s,         \
+                       (const u32x4 *)y, (const MAPT *)mappings, weights, (u32x4 *)out, T, k, R, vecs, nseg)
 #define DMOE_COMBINE_LAUNCH(MAPT, HALF, MODE)                                                                       \
-    hipLaunchKernelGGL((combine_kernel<MAPT, HALF, MODE>), dim3((unsigned)nblk), dim3(kBlock), 0, s, (const u32x4 *)y, \
-                       (const MAPT *)mappings, weights, (u32x4 *)out, T, k, R, vecs, nseg)
+    do {                                                                                                            \
+        if (streamed) DMOE_COMBINE_LAUNCH_ONE(MAPT, HALF, MODE, true);                                              \
+        else DMOE_COMBINE_LAUNCH_ONE(MAPT, HALF, MODE, false);                                                      \
+    } while (0)
     const bool half = dtype == DMOE_FP16;
     if (map_type == DMOE_I64) {
         if (!half && mode == 0) DMOE_COMBINE_LAUNCH(int64_t, false, 0);
@@ -380,6 +389,7 @@ extern "C" int dmoe_combine(const void *y, const void *mappings, int map_type, c
         else DMOE_COMBINE_LAUNCH(int32_t, true, 1);
     }
 #undef DMOE_COMBINE_LAUNCH
+#undef DMOE_COMBINE_LAUNCH_ONE
     DMOE_LAUNCH_CHECK("combine_kernel");
     return DMOE_OK;
 }

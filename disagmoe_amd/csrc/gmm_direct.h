@@ -16,6 +16,7 @@
 //   * 8 wavefronts (two per SIMD) on the 256-row tile, each with 128x64 of it; 4 wavefronts on the smaller tiles
 //     (64x128 of a 128-row tile, 64x64 of a 64-row tile); 32x32 v_mfma_f32_32x32x16_bf16 accumulators; operands are
 //     double buffered in registers one k-step ahead; one workgroup barrier per stage.
+#pragma once
 #include "gmm_common.h"
 
 namespace dmoe {
@@ -569,25 +570,6 @@ template <int kDM, int NW, int WM, int NP = 0>
 static int launch_direct_tile(const GmmArgs &args, bool trans_b, bool swiglu, hipStream_t stream) {
     if (trans_b) return swiglu ? launch_direct_one<kDM, NW, WM, true, true, false, NP>(args, stream) : launch_direct_one<kDM, NW, WM, true, false, false, NP>(args, stream);
     return swiglu ? launch_direct_one<kDM, NW, WM, false, true, false, NP>(args, stream) : launch_direct_one<kDM, NW, WM, false, false, false, NP>(args, stream);
-}
-
-// Preconditions (checked by the caller): bf16, K % 32 == 0, N % 8 == 0, K * N * 2 < 2^32.
-// tile_rows: 256 (8 wavefronts), 128 (4 wavefronts) or 64 (4 computing + 2 copying wavefronts); 260 = 256 rows on 4
-// wavefronts (comparison).
-int launch_direct_bf16(const GmmArgs &args, int tile_rows, bool trans_b, bool swiglu, hipStream_t stream) {
-    if (tile_rows == 64) return launch_direct_tile<64, 4, 1, 2>(args, trans_b, swiglu, stream);   // 4 + 2 copying wavefronts
-    if (tile_rows == 128) return launch_direct_tile<128, 4, 2>(args, trans_b, swiglu, stream);
-    if (tile_rows == 260) return launch_direct_tile<256, 4, 2>(args, trans_b, swiglu, stream);   // 256 rows on 4 wavefronts
-    return launch_direct_tile<256, 8, 2>(args, trans_b, swiglu, stream);
-}
-
-// Preconditions: e4m3 operands, K-contiguous on both sides, K % 64 == 0, N % 8 == 0, K * N < 2^32.
-int launch_direct_fp8(const GmmArgs &args, int tile_rows, bool swiglu, hipStream_t stream) {
-    if (tile_rows == 64) return swiglu ? launch_direct_one<64, 4, 1, true, true, true>(args, stream) : launch_direct_one<64, 4, 1, true, false, true>(args, stream);
-    // 256-row tiles: on 4 wavefronts they would need 256 accumulator + 96 operand registers per lane plus addressing;
-    // on 8 wavefronts a wavefront holds 128 + 48
-    if (tile_rows == 256) return swiglu ? launch_direct_one<256, 8, 2, true, true, true>(args, stream) : launch_direct_one<256, 8, 2, true, false, true>(args, stream);
-    return swiglu ? launch_direct_one<128, 4, 2, true, true, true>(args, stream) : launch_direct_one<128, 4, 2, true, false, true>(args, stream);
 }
 
 }  // namespace dmoe

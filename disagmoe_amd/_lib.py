@@ -28,6 +28,7 @@ SIGNATURES = {
     "dmoe_sort_by_prefill_order": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_void_p]),
     "dmoe_move_row_infos": (c_int, [c_void_p, c_int, c_void_p, c_int64, c_void_p]),
     "dmoe_expert_batch_sizes": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_int, c_void_p]),
+    "dmoe_host_mappings": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_void_p]),
     "dmoe_permute": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int, c_void_p,
                              c_void_p]),
     "dmoe_gather_rows": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int, c_void_p]),

@@ -63,3 +63,20 @@ extern "C" int dmoe_expert_batch_sizes(const int32_t *exp_ids, int64_t n, int n_
     }
     return DMOE_OK;
 }
+
+extern "C" int dmoe_host_mappings(const int32_t *exp_ids, int64_t n, int n_expert, int64_t *mappings, int64_t *exp_cnt) {
+    DMOE_REQUIRE(n >= 0 && n_expert > 0, DMOE_ERR_SHAPE, "dmoe_host_mappings: n=%lld n_expert=%d", (long long)n, n_expert);
+    DMOE_REQUIRE(n == 0 || (exp_ids && mappings), DMOE_ERR_ARG, "dmoe_host_mappings: null pointer");
+    std::vector<int64_t> cursor((size_t)n_expert, 0);
+    for (int64_t i = 0; i < n; ++i) {
+        DMOE_REQUIRE(exp_ids[i] >= 0 && exp_ids[i] < n_expert, DMOE_ERR_ARG, "dmoe_host_mappings: exp_ids[%lld]=%d outside [0, %d)",
+                     (long long)i, exp_ids[i], n_expert);
+        cursor[(size_t)exp_ids[i]] += 1;
+    }
+    if (exp_cnt)
+        for (int e = 0; e < n_expert; ++e) exp_cnt[e] = cursor[(size_t)e];
+    for (int e = 1; e < n_expert; ++e) cursor[(size_t)e] += cursor[(size_t)e - 1];   // end of every expert's rows
+    // rows of an expert are handed out from its last slot backwards, in the order the rows arrive
+    for (int64_t i = 0; i < n; ++i) mappings[i] = --cursor[(size_t)exp_ids[i]];
+    return DMOE_OK;
+}

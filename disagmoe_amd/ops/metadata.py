@@ -62,6 +62,16 @@ def expert_batch_sizes(exp_ids: Sequence[int], n_expert: int,
     return out.tolist()
 
 
+def host_mappings(exp_ids: Sequence[int], n_expert: int):
+    """``(mappings, exp_cnt)`` of the reference's counting sort (memory.py:38-52, datatypes.hpp:303-324)
+    computed on the host lists: experts ascending, inside an expert the first row takes the last slot."""
+    ids = _i32(exp_ids)
+    mappings = np.empty(ids.size, dtype=np.int64)
+    cnt = np.empty(n_expert, dtype=np.int64)
+    _lib.call("dmoe_host_mappings", _ptr(ids), ids.size, n_expert, _ptr(mappings), _ptr(cnt))
+    return mappings.tolist(), cnt.tolist()
+
+
 @dataclass
 class Metadata:
     """Field names and method names of the reference's ``Metadata`` as the expert step uses them."""
@@ -133,3 +143,57 @@ class Metadata:
         if topk == 1:
             return
         self.shape = [self.shape[0] // topk] + list(self.shape[1:])
+
+    @staticmethod
+    def merge_by_exp_ids(metas: Sequence["Metadata"], n_expert: Optional[int] = None):
+        """datatypes.hpp:287-337: the batches are concatenated and sorted by expert id with the rule of
+        ``host_mappings``; returns ``(merged, mappings)`` with ``mappings[idx]`` = row of the idx-th
+        incoming row in the merged batch.  ``n_expert`` defaults to the largest id + 1 (the reference
+        sizes its table for 32 experts)."""
+        assert len(metas) > 0
+        cat = lambda name: [v for m in metas for v in getattr(m, name)]
+        exp_ids = cat("exp_ids")
+        total = sum(m.num_tokens() for m in metas)
+        assert len(exp_ids) == total
+        if n_expert is None:
+            n_expert = max(exp_ids) + 1 if exp_ids else 1
+        mappings, _ = host_mappings(exp_ids, n_expert)
+        # the merged batch always carries one weight per row; batches without weights contribute zeros (:301, :327-329)
+        weights = [w for m in metas for w in (m.topk_weights if len(m.topk_weights) else [0.0] * m.num_tokens())]
+        merged = Metadata(shape=[total] + list(metas[0].shape[1:]), dtype=metas[0].dtype, layer_id=metas[0].layer_id,
+                          req_ids=move_row_infos(cat("req_ids"), mappings) if total else [],
+                          exp_ids=move_row_infos(exp_ids, mappings) if total else [],
+                          attn_dp_ranks=move_row_infos(cat("attn_dp_ranks"), mappings) if total else [],
+                          init_prefill_lens=move_row_infos(cat("init_prefill_lens"), mappings) if total else [],
+                          topk_weights=move_row_infos(weights, mappings, dtype=np.float32) if total else [])
+        return merged, mappings
+
+
+@dataclass
+class TensorBatch:
+    """Rows on the device with their bookkeeping (datatypes.hpp:503-506)."""
+    data: "torch.Tensor"
+    metadata: Metadata
+
+    @staticmethod
+    def merge(batches: Sequence["TensorBatch"], n_expert: Optional[int] = None) -> "TensorBatch":
+        """The expert worker's merge of the batches it received (datatypes.hpp:508-549): metadata by
+        ``merge_by_exp_ids``, rows gathered through a table of row pointers.  The table is built on the
+        device (one address per incoming row, scattered by the mapping), so nothing waits for the
+        stream, where the reference fills it in a host loop and synchronises after the gather
+        (csrc/cuda_ops/permute.cu:151).  The incoming tensors must stay alive until the gather has run."""
+        import torch
+        from . import memory
+        assert len(batches) > 0
+        meta, mappings = Metadata.merge_by_exp_ids([b.metadata for b in batches], n_expert)
+        first = batches[0].data
+        dev, hidden, dtype = first.device, first.shape[1], first.dtype
+        row_bytes = hidden * first.element_size()
+        addrs = []
+        for b in batches:
+            assert b.data.is_contiguous() and b.data.shape[1] == hidden and b.data.dtype == dtype
+            assert b.data.shape[0] == b.metadata.num_tokens()
+            addrs.append(b.data.data_ptr() + torch.arange(b.data.shape[0], dtype=torch.int64, device=dev) * row_bytes)
+        table = torch.empty(meta.num_tokens(), dtype=torch.int64, device=dev)
+        table[torch.tensor(mappings, dtype=torch.int64).to(dev, non_blocking=True)] = torch.cat(addrs)
+        return TensorBatch(memory.gather_row_ptrs(table, hidden, dtype), meta)

@@ -117,6 +117,12 @@ int dmoe_sort_by_prefill_order(const int32_t *req_ids, const int32_t *attn_dp_ra
 int dmoe_move_row_infos(const void *values, int elem_bytes, const int64_t *mapping, int64_t n, void *out);
 int dmoe_expert_batch_sizes(const int32_t *exp_ids, int64_t n, int n_expert, const int32_t *inner_exp_rank, int m,
                             int64_t *batches);
+/* The counting sort of Metadata::merge_by_exp_ids (csrc/include/datatypes.hpp:303-324) and of
+ * get_mappings_from_exp_ids (disagmoe/ops/memory.py:38-52) on host arrays: mappings[i] = destination row of
+ * row i of the concatenated batches, experts ascending, inside an expert the first row that arrives takes the
+ * last slot; exp_cnt[n_expert] (may be NULL) = rows per expert.  Any number of experts (the reference's table
+ * holds 32).  dmoe_route is the device form of the same rule. */
+int dmoe_host_mappings(const int32_t *exp_ids, int64_t n, int n_expert, int64_t *mappings, int64_t *exp_cnt);
 
 /* ---- row movement -------------------------------------------------------
  * dmoe_permute replaces permute_tokens_cuda(tokens, mappings, stream)

@@ -173,3 +173,25 @@ def test_row_buffers_beyond_4gib():
     first = torch.zeros(T, k, device=dev())
     first[:, 0] = 1
     assert torch.equal(memory.combine_tokens(p, m, first), x)
+
+
+def test_tensor_batch_merge():
+    # TensorBatch::merge (csrc/include/datatypes.hpp:508-549): rows of several incoming batches end up sorted by expert
+    from disagmoe_amd.ops.metadata import Metadata, TensorBatch
+    announce(test="tensor_batch_merge")
+    g = torch.Generator().manual_seed(21)
+    E, d = 8, 1024
+    batches, rows_all, ids_all = [], [], []
+    for n in (33, 1, 0, 250, 64):
+        ids = torch.randint(0, E, (n,), generator=g).tolist()
+        x = torch.randn(n, d, generator=g).to(torch.bfloat16)
+        rows_all.append(x)
+        ids_all.append(ids)
+        batches.append(TensorBatch(x.to(dev()), Metadata(shape=[n, d], req_ids=list(range(n)), exp_ids=ids)))
+    merged = TensorBatch.merge(batches, E)
+    m_ref, cnt = routing.merge_by_exp_ids(ids_all, E)
+    ref = torch.empty(sum(len(i) for i in ids_all), d, dtype=torch.bfloat16)
+    ref[torch.tensor(m_ref)] = torch.cat(rows_all)
+    assert torch.equal(merged.data.cpu(), ref)
+    assert merged.metadata.exp_ids == sorted(v for ids in ids_all for v in ids)
+    assert merged.metadata.get_expert_batch_sizes(E) == cnt

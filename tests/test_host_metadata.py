@@ -108,3 +108,42 @@ def test_metadata_topk_and_update():
     one.duplicate_topk(1)
     one.shrink_topk(1)
     assert one.shape == [2, 8] and one.req_ids == [1, 2]
+
+
+def test_host_mappings_known_answers_and_oracle(golden_dir):
+    for case in _load(golden_dir, "routing_kat.json")["cases"]:
+        m, cnt = metadata.host_mappings(case["ids"], case["E"])
+        assert m == case["mappings"] and cnt == case["exp_cnt"]
+    for n, E, seed in [(0, 3, 0), (1, 1, 1), (1000, 8, 2), (49152, 64, 3), (300, 100, 4)]:   # more than the reference's 32 experts
+        ids = np.random.default_rng(seed).integers(0, E, n).tolist()
+        m, cnt = metadata.host_mappings(ids, E)
+        m_ref, cnt_ref = routing.get_mappings_from_exp_ids(ids, E)
+        assert m == m_ref and cnt == cnt_ref
+    with pytest.raises(_lib.DmoeError):
+        metadata.host_mappings([0, 5], 5)
+
+
+def test_merge_by_exp_ids_matches_oracle():
+    rng = np.random.default_rng(12)
+    E = 6
+    metas, batches = [], []
+    base = 0
+    for n in (5, 0, 17, 9):
+        ids = rng.integers(0, E, n).tolist()
+        batches.append(ids)
+        metas.append(Metadata(shape=[n, 64], layer_id=3, req_ids=list(range(base, base + n)), exp_ids=ids,
+                              attn_dp_ranks=rng.integers(0, 2, n).tolist(), init_prefill_lens=rng.integers(-1, 9, n).tolist(),
+                              topk_weights=rng.random(n).astype(np.float32).tolist() if n != 9 else []))
+        base += n
+    merged, mappings = Metadata.merge_by_exp_ids(metas, E)
+    m_ref, cnt_ref = routing.merge_by_exp_ids(batches, E)
+    assert mappings == m_ref
+    cat = lambda name: [v for m in metas for v in getattr(m, name)]
+    assert merged.shape == [31, 64] and merged.layer_id == 3
+    assert merged.exp_ids == routing.apply_row_mapping(cat("exp_ids"), mappings) == sorted(cat("exp_ids"))
+    assert merged.req_ids == routing.apply_row_mapping(cat("req_ids"), mappings)
+    assert merged.attn_dp_ranks == routing.apply_row_mapping(cat("attn_dp_ranks"), mappings)
+    assert merged.init_prefill_lens == routing.apply_row_mapping(cat("init_prefill_lens"), mappings)
+    weights = cat("topk_weights") + [0.0] * 9      # the last batch came without weights
+    assert merged.topk_weights == routing.apply_row_mapping(weights, mappings)
+    assert merged.get_expert_batch_sizes(E) == cnt_ref

@@ -449,53 +449,60 @@ void gmm_direct_kernel(const GmmArgs p) {
         auto epilogue = [&]() {
             // ---- epilogue of the finished tile ----
             // The MFMAs take the B fragment as their first operand, so an accumulator holds the tile transposed:
-            // lane l owns output row l % 32 of its fragment and, in element x, column (x/4)*8 + (l/32)*4 + x%4.
-            // Four consecutive columns per lane -> one 8-byte store; a row is valid or not per lane.
+            // lane l owns output row l % 32 of its fragment and, in element x, column (x/4)*8 + (l/32)*4 + x%4:
+            // of every group of 8 columns the lower half of the wavefront holds the first 4, the upper half the last 4.
+            // Two groups at a time, the halves trade (v_permlane32_swap) what the other needs to own 8 consecutive
+            // columns: the lower half those of the first group, the upper half those of the second.  One 16-byte store
+            // per lane, 32 bytes per row and instruction; a row is valid or not for both lanes that share it.
             constexpr int FNO = SWIGLU ? FN / 2 : FN;
 #pragma unroll
             for (int i = 0; i < FM; ++i) {
                 const int r = wm * TM + i * 32 + l31;
                 if (r >= cur_rows_e) continue;
-                const int col_lane = cur_n0 + (SWIGLU ? wn * (TN / 2) : wn * TN) + kgrp * 4;
-                uint16_t *crow = (uint16_t *)p.c + (long long)(cur_row0 + r) * p.ldc + col_lane;
+                const int col0 = cur_n0 + (SWIGLU ? wn * (TN / 2) : wn * TN);
+                uint16_t *crow = (uint16_t *)p.c + (long long)(cur_row0 + r) * p.ldc + col0;
                 float sa = 1.f;
                 if constexpr (FP8) sa = p.a_scale[cur_row0 + r];
 #pragma unroll
                 for (int j = 0; j < FNO; ++j) {
 #pragma unroll
-                    for (int g = 0; g < 4; ++g) {
-                        const int col = col_lane + j * 32 + g * 8;
-                        if (col >= n_out) continue;   // n_out % 8 == 0: four columns at once
-                        float sb0[4] = {1.f, 1.f, 1.f, 1.f}, sb1[4] = {1.f, 1.f, 1.f, 1.f};
-                        if constexpr (FP8) {
-                            const float4 t0 = *(const float4 *)(p.b_scale + (long long)cur_e * p.N + col);
-                            sb0[0] = t0.x; sb0[1] = t0.y; sb0[2] = t0.z; sb0[3] = t0.w;
-                            if (SWIGLU) {
-                                const float4 t1 = *(const float4 *)(p.b_scale + (long long)cur_e * p.N + n_out + col);
-                                sb1[0] = t1.x; sb1[1] = t1.y; sb1[2] = t1.z; sb1[3] = t1.w;
-                            }
-                        }
-                        float v[4];
+                    for (int gp = 0; gp < 4; gp += 2) {
+                        uint2 pk[2];
 #pragma unroll
-                        for (int x = 0; x < 4; ++x) {
-                            if (SWIGLU) {
-                                const float gate = acc[i][j][g * 4 + x] * (sa * sb0[x]);
-                                v[x] = silu_mul(gate, acc[i][j + FN / 2][g * 4 + x] * (sa * sb1[x]));
-                            } else {
-                                v[x] = acc[i][j][g * 4 + x] * (sa * sb0[x]);
+                        for (int h = 0; h < 2; ++h) {
+                            const int g = gp + h;
+                            const int col = col0 + kgrp * 4 + j * 32 + g * 8;   // the 4 columns whose values this lane holds
+                            float sb0[4] = {1.f, 1.f, 1.f, 1.f}, sb1[4] = {1.f, 1.f, 1.f, 1.f};
+                            if constexpr (FP8) {
+                                if (col < n_out) {   // n_out % 8 == 0: a group of 8 columns is inside or outside as a whole
+                                    const float4 t0 = *(const float4 *)(p.b_scale + (long long)cur_e * p.N + col);
+                                    sb0[0] = t0.x; sb0[1] = t0.y; sb0[2] = t0.z; sb0[3] = t0.w;
+                                    if (SWIGLU) {
+                                        const float4 t1 = *(const float4 *)(p.b_scale + (long long)cur_e * p.N + n_out + col);
+                                        sb1[0] = t1.x; sb1[1] = t1.y; sb1[2] = t1.z; sb1[3] = t1.w;
+                                    }
+                                }
                             }
+                            float v[4];
+#pragma unroll
+                            for (int x = 0; x < 4; ++x) {
+                                if (SWIGLU) {
+                                    const float gate = acc[i][j][g * 4 + x] * (sa * sb0[x]);
+                                    v[x] = silu_mul(gate, acc[i][j + FN / 2][g * 4 + x] * (sa * sb1[x]));
+                                } else {
+                                    v[x] = acc[i][j][g * 4 + x] * (sa * sb0[x]);
+                                }
+                            }
+                            pk[h].x = pack_bf16x2(v[0], v[1]);
+                            pk[h].y = pack_bf16x2(v[2], v[3]);
                         }
-                        uint2 packed;
-                        packed.x = pack_bf16x2(v[0], v[1]);
-                        packed.y = pack_bf16x2(v[2], v[3]);
-#ifdef DMOE_DEBUG_HOOKS
-                        if (p.dbg == 7) {   // timing experiment: same bytes, fully coalesced addresses (wrong results)
-                            uint2 *lin = (uint2 *)((uint16_t *)p.c + (long long)cur_row0 * p.ldc) + ((wave * 64 + (i * FN * 4 + j * 4 + g)) * 64 + lane);
-                            *lin = packed;
-                            continue;
-                        }
-#endif
-                        *(uint2 *)(crow + j * 32 + g * 8) = packed;
+                        // lower half: [0] = its own part of group gp, [1] = the upper half's; upper half: [0] = the lower
+                        // half's part of group gp + 1, [1] = its own
+                        const auto lo = __builtin_amdgcn_permlane32_swap(pk[0].x, pk[1].x, false, false);
+                        const auto hi = __builtin_amdgcn_permlane32_swap(pk[0].y, pk[1].y, false, false);
+                        const int cst = j * 32 + (gp + kgrp) * 8;               // the 8 columns this lane stores
+                        if (col0 + cst >= n_out) continue;
+                        *(u32x4 *)(crow + cst) = u32x4{lo[0], hi[0], lo[1], hi[1]};
                     }
                 }
             }

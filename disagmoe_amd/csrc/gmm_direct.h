@@ -455,14 +455,37 @@ void gmm_direct_kernel(const GmmArgs p) {
             // columns: the lower half those of the first group, the upper half those of the second.  One 16-byte store
             // per lane, 32 bytes per row and instruction; a row is valid or not for both lanes that share it.
             constexpr int FNO = SWIGLU ? FN / 2 : FN;
+            const int col0 = cur_n0 + (SWIGLU ? wn * (TN / 2) : wn * TN);
+            // fp8 on 8 wavefronts: every scale this lane needs is fetched up front, all loads in flight together.  Rows
+            // and columns outside the tile read a valid neighbour; their results are never stored.  (On 4 wavefronts the
+            // registers for that are not there: the loads stay inside the loops.)
+            constexpr bool kScalesUpFront = FP8 && NW == 8;
+            float sa_all[kScalesUpFront ? FM : 1];
+            float4 sb_all[kScalesUpFront ? FNO * 4 * (SWIGLU ? 2 : 1) : 1];
+            if constexpr (kScalesUpFront) {
+#pragma unroll
+                for (int i = 0; i < FM; ++i) {
+                    const int r = wm * TM + i * 32 + l31;
+                    sa_all[i] = p.a_scale[cur_row0 + (r < cur_rows_e ? r : 0)];
+                }
+#pragma unroll
+                for (int j = 0; j < FNO; ++j)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        const int col = col0 + kgrp * 4 + j * 32 + g * 8;
+                        const float *sb = p.b_scale + (long long)cur_e * p.N + (col < n_out ? col : cur_n0);
+                        sb_all[(j * 4 + g) * (SWIGLU ? 2 : 1)] = *(const float4 *)sb;
+                        if (SWIGLU) sb_all[(j * 4 + g) * 2 + 1] = *(const float4 *)(sb + n_out);
+                    }
+            }
 #pragma unroll
             for (int i = 0; i < FM; ++i) {
                 const int r = wm * TM + i * 32 + l31;
                 if (r >= cur_rows_e) continue;
-                const int col0 = cur_n0 + (SWIGLU ? wn * (TN / 2) : wn * TN);
                 uint16_t *crow = (uint16_t *)p.c + (long long)(cur_row0 + r) * p.ldc + col0;
                 float sa = 1.f;
-                if constexpr (FP8) sa = p.a_scale[cur_row0 + r];
+                if constexpr (kScalesUpFront) sa = sa_all[i];
+                else if constexpr (FP8) sa = p.a_scale[cur_row0 + r];
 #pragma unroll
                 for (int j = 0; j < FNO; ++j) {
 #pragma unroll
@@ -471,9 +494,16 @@ void gmm_direct_kernel(const GmmArgs p) {
 #pragma unroll
                         for (int h = 0; h < 2; ++h) {
                             const int g = gp + h;
-                            const int col = col0 + kgrp * 4 + j * 32 + g * 8;   // the 4 columns whose values this lane holds
                             float sb0[4] = {1.f, 1.f, 1.f, 1.f}, sb1[4] = {1.f, 1.f, 1.f, 1.f};
-                            if constexpr (FP8) {
+                            if constexpr (kScalesUpFront) {
+                                const float4 t0 = sb_all[(j * 4 + g) * (SWIGLU ? 2 : 1)];
+                                sb0[0] = t0.x; sb0[1] = t0.y; sb0[2] = t0.z; sb0[3] = t0.w;
+                                if (SWIGLU) {
+                                    const float4 t1 = sb_all[(j * 4 + g) * 2 + 1];
+                                    sb1[0] = t1.x; sb1[1] = t1.y; sb1[2] = t1.z; sb1[3] = t1.w;
+                                }
+                            } else if constexpr (FP8) {
+                                const int col = col0 + kgrp * 4 + j * 32 + g * 8;   // the 4 columns whose values this lane holds
                                 if (col < n_out) {   // n_out % 8 == 0: a group of 8 columns is inside or outside as a whole
                                     const float4 t0 = *(const float4 *)(p.b_scale + (long long)cur_e * p.N + col);
                                     sb0[0] = t0.x; sb0[1] = t0.y; sb0[2] = t0.z; sb0[3] = t0.w;

@@ -305,6 +305,10 @@ void gmm_direct_kernel(const GmmArgs p) {
         }
     }
 
+#ifdef DMOE_DEBUG_HOOKS
+    unsigned long long dbg_sum[6] = {0, 0, 0, 0, 0, 0}, dbg_t[5] = {0, 0, 0, 0, 0};
+    const bool dbg_rec = (p.dbg == 21 || p.dbg == 22) && blockIdx.x == 8;
+#endif
     while (q < total) {
         // results of this tile go here after the next tile's copies have been issued
         const int cur_row0 = row0, cur_rows_e = rows_e, cur_n0 = n0, cur_e = e;
@@ -339,8 +343,14 @@ void gmm_direct_kernel(const GmmArgs p) {
 
         // stage 0 of this tile has landed (its other prologue stages, and stores of the previous tile's
         // epilogue that were issued after them, may still be in flight: waiting for fewer is only stricter)
+#ifdef DMOE_DEBUG_HOOKS
+        if (dbg_rec) dbg_t[0] = __builtin_amdgcn_s_memtime();
+#endif
         if constexpr (NP == 0) wait_ahead(pre - 1);
         __syncthreads();
+#ifdef DMOE_DEBUG_HOOKS
+        if (dbg_rec) dbg_t[1] = __builtin_amdgcn_s_memtime();
+#endif
 #pragma unroll
         for (int r = 0; r < NR; ++r) load_frag(0, 0, 0, r);
 
@@ -387,6 +397,9 @@ void gmm_direct_kernel(const GmmArgs p) {
                 else wait_ahead(ahead);
                 __syncthreads();
                 __builtin_amdgcn_sched_barrier(0);
+#ifdef DMOE_DEBUG_HOOKS
+                if (dbg_rec && (s == 0 || s == 3)) dbg_t[s == 0 ? 2 : 3] = __builtin_amdgcn_s_memtime();
+#endif
             }
             static_for<0, NM>([&](auto t_tag) {
                 constexpr int t = decltype(t_tag)::value;
@@ -446,6 +459,9 @@ void gmm_direct_kernel(const GmmArgs p) {
             q = s_item;        // the next work item, written by them before the barrier
         }
 
+#ifdef DMOE_DEBUG_HOOKS
+        if (dbg_rec) dbg_t[4] = __builtin_amdgcn_s_memtime();
+#endif
         auto epilogue = [&]() {
             // ---- epilogue of the finished tile ----
             // The MFMAs take the B fragment as their first operand, so an accumulator holds the tile transposed:
@@ -478,14 +494,26 @@ void gmm_direct_kernel(const GmmArgs p) {
                         if (SWIGLU) sb_all[(j * 4 + g) * 2 + 1] = *(const float4 *)(sb + n_out);
                     }
             }
+            // Beside computing-only kernels the 16-byte pieces then pass through LDS (the stage buffer after the last
+            // stage's, private 4 KiB per wavefront, free until the next tile's copies are issued behind the barrier that
+            // follows): a block of 32 rows x 64 (or 32) columns goes in by row of the fragment and comes out by row of
+            // the result, so that a store instruction writes 8 whole rows of 128 bytes (16 of 64), not 32 pieces of 32.
+            // Chunks are placed at chunk ^ (row & 7) (or & 3): the writes and the reads are free of bank conflicts.
+            constexpr bool kViaLds = NP == 0;
+            constexpr int CW = FNO >= 2 ? 2 : 1;          // fragments (of 32 columns) staged together
+            constexpr int RB = CW * 64;                   // bytes per staged row
+            constexpr int CPR = RB / 16;                  // 16-byte chunks per row = lanes that write a row out
+            constexpr int RPI = 64 / CPR;                 // rows per store instruction
+            char *stg = smem + (S % kStages) * kStage + wave * 4096;
 #pragma unroll
             for (int i = 0; i < FM; ++i) {
                 const int r = wm * TM + i * 32 + l31;
-                if (r >= cur_rows_e) continue;
+                const bool row_ok = r < cur_rows_e;
+                if (!kViaLds && !row_ok) continue;
                 uint16_t *crow = (uint16_t *)p.c + (long long)(cur_row0 + r) * p.ldc + col0;
                 float sa = 1.f;
                 if constexpr (kScalesUpFront) sa = sa_all[i];
-                else if constexpr (FP8) sa = p.a_scale[cur_row0 + r];
+                else if constexpr (FP8) sa = p.a_scale[cur_row0 + (row_ok ? r : 0)];
 #pragma unroll
                 for (int j = 0; j < FNO; ++j) {
 #pragma unroll
@@ -530,9 +558,31 @@ void gmm_direct_kernel(const GmmArgs p) {
                         // half's part of group gp + 1, [1] = its own
                         const auto lo = __builtin_amdgcn_permlane32_swap(pk[0].x, pk[1].x, false, false);
                         const auto hi = __builtin_amdgcn_permlane32_swap(pk[0].y, pk[1].y, false, false);
-                        const int cst = j * 32 + (gp + kgrp) * 8;               // the 8 columns this lane stores
-                        if (col0 + cst >= n_out) continue;
-                        *(u32x4 *)(crow + cst) = u32x4{lo[0], hi[0], lo[1], hi[1]};
+                        const u32x4 piece = {lo[0], hi[0], lo[1], hi[1]};
+                        if constexpr (kViaLds) {
+                            const int cidx = (j % CW) * 4 + gp + kgrp;          // chunk of the staged row this lane holds
+                            *(u32x4 *)(stg + l31 * RB + ((cidx ^ (l31 & (CPR - 1))) << 4)) = piece;
+                            if ((j % CW) == CW - 1 && gp == 2) {
+                                // the block is complete: out by rows
+#pragma unroll
+                                for (int q = 0; q < 32 / RPI; ++q) {
+                                    const int row = q * RPI + lane / CPR, c = lane % CPR;
+                                    const u32x4 val = *(const u32x4 *)(stg + row * RB + ((c ^ (row & (CPR - 1))) << 4));
+                                    const int grow = wm * TM + i * 32 + row;
+                                    const int gcol = col0 + (j - (CW - 1)) * 32 + c * 8;
+                                    if (grow >= cur_rows_e || gcol >= n_out) continue;
+#ifdef DMOE_DEBUG_HOOKS
+                                    // timing experiment 8: the epilogue without its stores (a value that never occurs)
+                                    if (p.dbg == 8 && val[0] != 0x7fc17fc1u) continue;
+#endif
+                                    *(u32x4 *)((uint16_t *)p.c + (long long)(cur_row0 + grow) * p.ldc + gcol) = val;
+                                }
+                            }
+                        } else {
+                            const int cst = j * 32 + (gp + kgrp) * 8;           // the 8 columns this lane stores
+                            if (col0 + cst >= n_out) continue;
+                            *(u32x4 *)(crow + cst) = piece;
+                        }
                     }
                 }
             }
@@ -541,7 +591,22 @@ void gmm_direct_kernel(const GmmArgs p) {
 #ifdef DMOE_DEBUG_HOOKS
         if (p.dbg == 6) return;   // timing experiment: results not stored
 #endif
+#ifdef DMOE_DEBUG_HOOKS
+        if (p.dbg == 22) {}   // timing experiment: where the time of a tile goes, without the epilogue
+        else
+#endif
         epilogue();
+#ifdef DMOE_DEBUG_HOOKS
+        if (dbg_rec) {
+            const unsigned long long t5 = __builtin_amdgcn_s_memtime();
+            dbg_sum[0] += dbg_t[1] - dbg_t[0];   // wait for stage 0
+            dbg_sum[1] += dbg_t[2] - dbg_t[1];   // stage 0 up to its hand-over
+            dbg_sum[2] += dbg_t[3] - dbg_t[2];   // stages 1 .. 3
+            dbg_sum[3] += dbg_t[4] - dbg_t[3];   // rest of the main loop
+            dbg_sum[4] += t5 - dbg_t[4];         // epilogue
+            dbg_sum[5] += 1;
+        }
+#endif
         };   // run_tile
         // fp8: one instance per wavefront number (the MFMA slots of its copies are compile-time constants)
         auto run_build = [&](auto guard_tag) {
@@ -576,6 +641,12 @@ void gmm_direct_kernel(const GmmArgs p) {
         if constexpr (NP == 0) next_item();
         else if (q < total) locate_tile(q);
     }
+#ifdef DMOE_DEBUG_HOOKS
+    if (dbg_rec && tid == 0 && dbg_sum[5] > 0)
+        printf("[dbg %d] tiles %llu; per tile (clk): wait for stage 0 %llu, stage 0 %llu, stages 1-3 %llu, rest of the loop %llu, epilogue %llu\n",
+               p.dbg, dbg_sum[5], dbg_sum[0] / dbg_sum[5], dbg_sum[1] / dbg_sum[5], dbg_sum[2] / dbg_sum[5],
+               dbg_sum[3] / dbg_sum[5], dbg_sum[4] / dbg_sum[5]);
+#endif
     sched_finish(p.sched_slot);
 }
 

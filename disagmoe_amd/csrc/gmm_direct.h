@@ -498,13 +498,15 @@ void gmm_direct_kernel(const GmmArgs p) {
             // stage's, private 4 KiB per wavefront, free until the next tile's copies are issued behind the barrier that
             // follows): a block of 32 rows x 64 (or 32) columns goes in by row of the fragment and comes out by row of
             // the result, so that a store instruction writes 8 whole rows of 128 bytes (16 of 64), not 32 pieces of 32.
-            // Chunks are placed at chunk ^ (row & 7) (or & 3): the writes and the reads are free of bank conflicts.
+            // Chunks are placed at chunk ^ (row & 7) (128-byte rows) or chunk ^ ((row >> 1) & 3) (64-byte rows, two to a
+            // line of banks): the writes and the reads are free of bank conflicts.
             constexpr bool kViaLds = NP == 0;
             constexpr int CW = FNO >= 2 ? 2 : 1;          // fragments (of 32 columns) staged together
             constexpr int RB = CW * 64;                   // bytes per staged row
             constexpr int CPR = RB / 16;                  // 16-byte chunks per row = lanes that write a row out
             constexpr int RPI = 64 / CPR;                 // rows per store instruction
             char *stg = smem + (S % kStages) * kStage + wave * 4096;
+            auto swz = [](int row) { return CPR == 8 ? (row & 7) : ((row >> 1) & 3); };
 #pragma unroll
             for (int i = 0; i < FM; ++i) {
                 const int r = wm * TM + i * 32 + l31;
@@ -561,13 +563,13 @@ void gmm_direct_kernel(const GmmArgs p) {
                         const u32x4 piece = {lo[0], hi[0], lo[1], hi[1]};
                         if constexpr (kViaLds) {
                             const int cidx = (j % CW) * 4 + gp + kgrp;          // chunk of the staged row this lane holds
-                            *(u32x4 *)(stg + l31 * RB + ((cidx ^ (l31 & (CPR - 1))) << 4)) = piece;
+                            *(u32x4 *)(stg + l31 * RB + ((cidx ^ swz(l31)) << 4)) = piece;
                             if ((j % CW) == CW - 1 && gp == 2) {
                                 // the block is complete: out by rows
 #pragma unroll
                                 for (int q = 0; q < 32 / RPI; ++q) {
                                     const int row = q * RPI + lane / CPR, c = lane % CPR;
-                                    const u32x4 val = *(const u32x4 *)(stg + row * RB + ((c ^ (row & (CPR - 1))) << 4));
+                                    const u32x4 val = *(const u32x4 *)(stg + row * RB + ((c ^ swz(row)) << 4));
                                     const int grow = wm * TM + i * 32 + row;
                                     const int gcol = col0 + (j - (CW - 1)) * 32 + c * 8;
                                     if (grow >= cur_rows_e || gcol >= n_out) continue;

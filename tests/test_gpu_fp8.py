@@ -133,3 +133,24 @@ def test_c5_full_size_sampled():
     assert worst <= TOL_FP8, worst
     assert noise <= TOL_FP8_ACT, noise
     assert torch.isfinite(out.float()).all()
+
+
+@pytest.mark.parametrize("variant", [0, 5, 6, 7])
+@pytest.mark.parametrize("K", [64, 128])
+def test_gmm_fp8_few_stages(variant, K):
+    announce(test="gmm_fp8_few_stages", variant=variant, K=K)
+    gg.set_tile_variant(variant)
+    try:
+        E, R, N = 3, 700, 512
+        g = torch.Generator().manual_seed(K)
+        a = torch.randn(R, K, generator=g).to(torch.bfloat16)
+        w = (torch.randn(E, K, N, generator=g) * 0.05).to(torch.bfloat16)
+        sizes = ragged_sizes(E, R, seed=K)
+        aq, a_s = fp8.quantize_rows(a)
+        wq, w_s = fp8.quantize_weight_channels(w)
+        out = gg.gmm_fp8(aq.to(dev()), a_s.to(dev()), wq.to(dev()), w_s.to(dev()), sizes)
+        exact = ffn.gmm(fp8.dequantize_rows(aq, a_s, torch.float32), fp8.dequantize_weight(wq, w_s, torch.float32), sizes,
+                        out_dtype=torch.float32)
+        assert max_rel_err(out, exact) <= TOL_FP8
+    finally:
+        gg.set_tile_variant(0)

@@ -187,3 +187,22 @@ def test_gmm_weights_beyond_32bit_offsets(trans_b):
     ref = ffn.gmm(a, b_cols, sizes)
     assert max_rel_err(out[:, cols.to(dev())], ref) <= TOL_BF16
     assert torch.isfinite(out.float()).all()
+
+
+@pytest.mark.parametrize("variant", [0, 5, 6, 7])
+@pytest.mark.parametrize("K", [32, 64, 96])
+def test_gmm_few_stages(variant, K):
+    # one, two and three 32-k stages: fewer than the LDS pipeline is deep (its prologue, tail and the staging of the
+    # results in a free stage buffer all take their short paths)
+    announce(test="gmm_few_stages", variant=variant, K=K)
+    gg.set_tile_variant(variant)
+    E, R, N = 3, 700, 512
+    sizes = ragged_sizes(E, R, seed=K)
+    a = _rand((R, K), 41)
+    b = _rand((E, K, N), 42, std=0.1)
+    out = gg.gmm(a.to(dev()), b.to(dev()), sizes)
+    assert max_rel_err(out, ffn.gmm(a, b, sizes)) <= TOL_BF16
+    w13 = _rand((E, K, 2 * N), 43, std=0.1)
+    up = ffn.gmm(a, w13, sizes, out_dtype=torch.float32)
+    ref = torch.nn.functional.silu(up[:, :N]) * up[:, N:]
+    assert max_rel_err(gg.gmm_swiglu(a.to(dev()), w13.to(dev()), sizes), ref) <= TOL_BF16

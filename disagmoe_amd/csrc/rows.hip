@@ -193,24 +193,6 @@ __global__ __launch_bounds__(kBlock) void combine_kernel(const u32x4 *__restrict
     }
 }
 
-// fp32 -> OCP e4m3fn, round to nearest even, saturating at +-448.
-__device__ __forceinline__ uint32_t f32_to_e4m3(float f) {
-    const uint32_t u = __float_as_uint(f);
-    const uint32_t sign = (u >> 24) & 0x80u;
-    float a = fabsf(f);
-    if (!(a == a)) return sign | 0x7fu;  // NaN
-    if (a >= 448.f) return sign | 0x7eu; // saturate (also covers inf)
-    if (a < 0.015625f) {                 // below 2^-6: subnormal grid of 2^-9
-        const float q = rintf(a * 512.f);  // round half to even
-        return sign | (uint32_t)q;         // q == 8 encodes 2^-6, the first normal
-    }
-    uint32_t bits = __float_as_uint(a);
-    bits += 0x7ffffu + ((bits >> 20) & 1u);  // round to 3 mantissa bits, ties to even
-    const uint32_t exp = (bits >> 23) - 127 + 7;
-    const uint32_t man = (bits >> 20) & 7u;
-    return sign | (exp << 3) | man;
-}
-
 // q[r,:] = fp8(x[r,:] / s[r]), s[r] = absmax / 448.  One workgroup per row.
 template <bool kHalf>
 __global__ __launch_bounds__(kBlock) void quant_rows_kernel(const u32x4 *__restrict__ x, uint2 *__restrict__ q,
@@ -243,9 +225,12 @@ __global__ __launch_bounds__(kBlock) void quant_rows_kernel(const u32x4 *__restr
         uint32_t o[2] = {0, 0};
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const float lo = elem_to_f32<kHalf>((uint16_t)(b[i] & 0xffffu)) / s;
-            const float hi = elem_to_f32<kHalf>((uint16_t)(b[i] >> 16)) / s;
-            o[i / 2] |= (f32_to_e4m3(lo) | (f32_to_e4m3(hi) << 8)) << (16 * (i & 1));
+            // the hardware conversion (OCP e4m3fn on gfx950, round to nearest even) of the pair, after the clamp to the
+            // largest finite value that the division can overshoot by an ulp
+            const float lo = __builtin_amdgcn_fmed3f(elem_to_f32<kHalf>((uint16_t)(b[i] & 0xffffu)) / s, -448.f, 448.f);
+            const float hi = __builtin_amdgcn_fmed3f(elem_to_f32<kHalf>((uint16_t)(b[i] >> 16)) / s, -448.f, 448.f);
+            if (i & 1) o[i / 2] = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(lo, hi, (int)o[i / 2], true);
+            else o[i / 2] = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(lo, hi, (int)o[i / 2], false);
         }
         dst[v] = make_uint2(o[0], o[1]);
     }

@@ -140,8 +140,12 @@ def main() -> int:
 
     def step():
         mappings, batch_sizes, _ = memory.route_tokens(ids, w.E)
-        permuted = memory.permute_tokens_cuda(x, mappings)
-        y = layer.forward(w.R, permuted, batch_sizes)
+        if w.fp8:   # the routed rows are quantised on their way into the expert-sorted buffer
+            xq, xs = memory.permute_quantize(x, mappings)
+            y = layer.forward_quantized(w.R, xq, xs, batch_sizes)
+        else:
+            permuted = memory.permute_tokens_cuda(x, mappings)
+            y = layer.forward(w.R, permuted, batch_sizes)
         return memory.combine_tokens(y, mappings, gates)
 
     if args.copy_probe_mib > 0:
@@ -177,8 +181,10 @@ def main() -> int:
         hq, hs = gg.quantize_rows(h)
         up_ms, _ = _event_ms(lambda: gg.gmm_fp8_swiglu(xq, xs, layer.w13_q, layer.w13_scale, batch_sizes, c=h), it)
         down_ms, _ = _event_ms(lambda: gg.gmm_fp8(hq, hs, layer.w2_q, layer.w2_scale, batch_sizes), it)
-        q_ms, _ = _event_ms(lambda: gg.quantize_rows(permuted), it)
-        stages["quant_rows"] = {"ms": q_ms}
+        q_ms, _ = _event_ms(lambda: gg.quantize_rows(h), it)
+        stages["quant_rows"] = {"ms": q_ms, "GB/s": 3.0 * w.R * w.I / q_ms / 1e6}       # the [R, I] intermediate
+        pq_ms, _ = _event_ms(lambda: memory.permute_quantize(x, mappings), it)
+        stages["permute_quantize"] = {"ms": pq_ms, "GB/s": (2.0 * w.T + w.R) * w.d / pq_ms / 1e6}   # bytes actually moved
         peak = PEAK_FP8_TFLOPS
         tile = _tile_rows(w)
         # mirrors the dispatch of launch_by_rows (csrc/gmm.hip): the global-to-LDS kernel takes whole 64-k stages

@@ -42,6 +42,8 @@ SIGNATURES = {
     "dmoe_gmm_workspace_bytes": (c_int, [c_int, POINTER(c_size_t)]),
     "dmoe_gmm_tune": (c_int, [c_int]),
     "dmoe_quant_rows": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int, c_void_p]),
+    "dmoe_permute_quant": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int,
+                                   c_void_p]),
     "dmoe_gmm_fp8": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int64,
                              c_int64, c_void_p]),
     "dmoe_gmm_fp8_swiglu": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int,

@@ -193,21 +193,37 @@ __global__ __launch_bounds__(kBlock) void combine_kernel(const u32x4 *__restrict
     }
 }
 
-// q[r,:] = fp8(x[r,:] / s[r]), s[r] = absmax / 448.  One workgroup per row.
-template <bool kHalf>
-__global__ __launch_bounds__(kBlock) void quant_rows_kernel(const u32x4 *__restrict__ x, uint2 *__restrict__ q,
-                                                           float *__restrict__ scales, int64_t rows, int vecs) {
+// q[map[i*k + j], :] = fp8(x[i, :] / s[i]) and scales[map[i*k + j]] = s[i] for j < k: the permute and the per-row
+// quantisation in one pass (without a mapping: the quantisation alone, q[i, :] and scales[i]).  One workgroup per token;
+// the row is read once (kept in registers when it has at most 16384 elements), quantised once and stored k times.
+template <typename MapT, bool kHalf>
+__global__ __launch_bounds__(kBlock) void permute_quant_kernel(const u32x4 *__restrict__ x, uint2 *__restrict__ q,
+                                                              float *__restrict__ scales, const MapT *__restrict__ map,
+                                                              int k, int64_t R, int vecs) {
+    constexpr int kKeep = 8;   // 16-byte vectors per thread held in registers
     __shared__ float wave_max[kBlock / kWave];
-    const int64_t r = blockIdx.x;
-    const u32x4 *src = x + r * vecs;
+    const int64_t tok = blockIdx.x;
+    const u32x4 *src = x + tok * vecs;
+    const bool keep = vecs <= kKeep * kBlock;
+    u32x4 held[kKeep];
     float amax = 0.f;
-    for (int v = threadIdx.x; v < vecs; v += kBlock) {
-        const u32x4 b = src[v];
+    auto absmax_of = [&](const u32x4 &b) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             amax = fmaxf(amax, fabsf(elem_to_f32<kHalf>((uint16_t)(b[i] & 0xffffu))));
             amax = fmaxf(amax, fabsf(elem_to_f32<kHalf>((uint16_t)(b[i] >> 16))));
         }
+    };
+    if (keep) {
+#pragma unroll
+        for (int u = 0; u < kKeep; ++u) {
+            const int v = threadIdx.x + u * kBlock;
+            held[u] = u32x4{0, 0, 0, 0};
+            if (v < vecs) held[u] = __builtin_nontemporal_load(src + v);
+            absmax_of(held[u]);
+        }
+    } else {
+        for (int v = threadIdx.x; v < vecs; v += kBlock) absmax_of(src[v]);
     }
 #pragma unroll
     for (int s = kWave / 2; s > 0; s >>= 1) amax = fmaxf(amax, __shfl_xor(amax, s, kWave));
@@ -218,21 +234,40 @@ __global__ __launch_bounds__(kBlock) void quant_rows_kernel(const u32x4 *__restr
     for (int i = 1; i < kBlock / kWave; ++i) amax = fmaxf(amax, wave_max[i]);
     float s = amax / 448.f;
     if (!(s > 0.f)) s = 1.f;
-    if (threadIdx.x == 0) scales[r] = s;
-    uint2 *dst = q + r * vecs;
-    for (int v = threadIdx.x; v < vecs; v += kBlock) {
-        const u32x4 b = src[v];
+    auto quantised = [&](const u32x4 &b) {
         uint32_t o[2] = {0, 0};
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            // the hardware conversion (OCP e4m3fn on gfx950, round to nearest even) of the pair, after the clamp to the
-            // largest finite value that the division can overshoot by an ulp
             const float lo = __builtin_amdgcn_fmed3f(elem_to_f32<kHalf>((uint16_t)(b[i] & 0xffffu)) / s, -448.f, 448.f);
             const float hi = __builtin_amdgcn_fmed3f(elem_to_f32<kHalf>((uint16_t)(b[i] >> 16)) / s, -448.f, 448.f);
             if (i & 1) o[i / 2] = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(lo, hi, (int)o[i / 2], true);
             else o[i / 2] = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(lo, hi, (int)o[i / 2], false);
         }
-        dst[v] = make_uint2(o[0], o[1]);
+        return make_uint2(o[0], o[1]);
+    };
+    if (keep) {
+        uint2 out[kKeep];
+#pragma unroll
+        for (int u = 0; u < kKeep; ++u) out[u] = quantised(held[u]);
+        for (int j = 0; j < k; ++j) {
+            const int64_t p = map ? load_map(map, tok * k + j) : tok;   // no mapping: rows stay where they are
+            if (p < 0 || p >= R) continue;
+            if (threadIdx.x == 0) scales[p] = s;
+            uint2 *dst = q + p * vecs;
+#pragma unroll
+            for (int u = 0; u < kKeep; ++u) {
+                const int v = threadIdx.x + u * kBlock;
+                if (v < vecs) dst[v] = out[u];
+            }
+        }
+    } else {
+        for (int j = 0; j < k; ++j) {
+            const int64_t p = map ? load_map(map, tok * k + j) : tok;   // no mapping: rows stay where they are
+            if (p < 0 || p >= R) continue;
+            if (threadIdx.x == 0) scales[p] = s;
+            uint2 *dst = q + p * vecs;
+            for (int v = threadIdx.x; v < vecs; v += kBlock) dst[v] = quantised(src[v]);
+        }
     }
 }
 
@@ -388,12 +423,38 @@ extern "C" int dmoe_quant_rows(const void *x, void *q, float *scales, int64_t ro
     DMOE_REQUIRE(rows >= 0 && rows < (1ll << 31), DMOE_ERR_ARG, "dmoe_quant_rows: bad row count");
     if (rows == 0) return DMOE_OK;
     DMOE_REQUIRE(x && q && scales, DMOE_ERR_ARG, "dmoe_quant_rows: null pointer");
+    // the fused permute + quantise kernel without a mapping
     if (dtype == DMOE_FP16)
-        hipLaunchKernelGGL((quant_rows_kernel<true>), dim3((unsigned)rows), dim3(kBlock), 0, (hipStream_t)stream,
-                           (const u32x4 *)x, (uint2 *)q, scales, rows, vecs);
+        hipLaunchKernelGGL((permute_quant_kernel<int64_t, true>), dim3((unsigned)rows), dim3(kBlock), 0, (hipStream_t)stream,
+                           (const u32x4 *)x, (uint2 *)q, scales, (const int64_t *)nullptr, 1, rows, vecs);
     else
-        hipLaunchKernelGGL((quant_rows_kernel<false>), dim3((unsigned)rows), dim3(kBlock), 0, (hipStream_t)stream,
-                           (const u32x4 *)x, (uint2 *)q, scales, rows, vecs);
-    DMOE_LAUNCH_CHECK("quant_rows_kernel");
+        hipLaunchKernelGGL((permute_quant_kernel<int64_t, false>), dim3((unsigned)rows), dim3(kBlock), 0, (hipStream_t)stream,
+                           (const u32x4 *)x, (uint2 *)q, scales, (const int64_t *)nullptr, 1, rows, vecs);
+    DMOE_LAUNCH_CHECK("permute_quant_kernel");
+    return DMOE_OK;
+}
+
+extern "C" int dmoe_permute_quant(const void *in, void *q, float *scales, const void *mappings, int map_type, int64_t T,
+                                  int64_t R, int64_t d, int dtype, void *stream) {
+    int vecs = 0;
+    int rc = check_rows("dmoe_permute_quant", d, dtype, &vecs);
+    if (rc != DMOE_OK) return rc;
+    DMOE_REQUIRE(dtype == DMOE_BF16 || dtype == DMOE_FP16, DMOE_ERR_DTYPE, "dmoe_permute_quant: dtype %d", dtype);
+    DMOE_REQUIRE(T >= 0 && R >= 0 && T < (1ll << 31), DMOE_ERR_ARG, "dmoe_permute_quant: bad T/R");
+    DMOE_REQUIRE(T == 0 ? R == 0 : R % T == 0, DMOE_ERR_SHAPE, "dmoe_permute_quant: R=%lld is not a multiple of T=%lld",
+                 (long long)R, (long long)T);
+    DMOE_REQUIRE(map_type == DMOE_I32 || map_type == DMOE_I64, DMOE_ERR_DTYPE, "dmoe_permute_quant: mapping type %d", map_type);
+    if (R == 0) return DMOE_OK;
+    DMOE_REQUIRE(in && q && scales && mappings, DMOE_ERR_ARG, "dmoe_permute_quant: null pointer");
+    const int k = (int)(R / T);
+    hipStream_t s = (hipStream_t)stream;
+#define DMOE_PQ_LAUNCH(MAPT, HALF)                                                                                     \
+    hipLaunchKernelGGL((permute_quant_kernel<MAPT, HALF>), dim3((unsigned)T), dim3(kBlock), 0, s, (const u32x4 *)in,   \
+                       (uint2 *)q, scales, (const MAPT *)mappings, k, R, vecs)
+    const bool half = dtype == DMOE_FP16;
+    if (map_type == DMOE_I64) { if (half) DMOE_PQ_LAUNCH(int64_t, true); else DMOE_PQ_LAUNCH(int64_t, false); }
+    else { if (half) DMOE_PQ_LAUNCH(int32_t, true); else DMOE_PQ_LAUNCH(int32_t, false); }
+#undef DMOE_PQ_LAUNCH
+    DMOE_LAUNCH_CHECK("permute_quant_kernel");
     return DMOE_OK;
 }

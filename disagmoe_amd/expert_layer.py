@@ -27,6 +27,11 @@ def expert_layer_forward(experts: torch.nn.Module, x: torch.Tensor, topk_ids: to
     T, k = topk_ids.shape
     num_experts = experts.num_experts
     mappings, batch_sizes, offsets = memory.route_tokens(topk_ids, num_experts, order)
+    if hasattr(experts, "forward_quantized") and stages is None:
+        # fp8 experts: the routed rows are quantised on their way into the expert-sorted buffer
+        xq, xs = memory.permute_quantize(x, mappings)
+        expert_out = experts.forward_quantized(T * k, xq, xs, batch_sizes)
+        return memory.combine_tokens(expert_out, mappings, topk_weights)
     permuted = memory.permute_tokens_cuda(x, mappings)
     expert_out = experts.forward(T * k, permuted, batch_sizes)
     out = memory.combine_tokens(expert_out, mappings, topk_weights)

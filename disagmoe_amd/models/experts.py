@@ -125,6 +125,10 @@ class MoEExpertsFP8(torch.nn.Module):
 
     def forward(self, bs: int, hiddens: torch.Tensor, batch_sizes: torch.Tensor) -> torch.Tensor:
         xq, xs = gg.quantize_rows(hiddens)
+        return self.forward_quantized(bs, xq, xs, batch_sizes)
+
+    def forward_quantized(self, bs: int, xq: torch.Tensor, xs: torch.Tensor, batch_sizes: torch.Tensor) -> torch.Tensor:
+        """The same on rows that arrive quantised (``ops.memory.permute_quantize``)."""
         h = gg.gmm_fp8_swiglu(xq, xs, self.w13_q, self.w13_scale, batch_sizes)
         hq, hs = gg.quantize_rows(h)
         return gg.gmm_fp8(hq, hs, self.w2_q, self.w2_scale, batch_sizes)

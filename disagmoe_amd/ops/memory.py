@@ -123,6 +123,26 @@ def permute_tokens_cuda(tokens: torch.Tensor, mappings: Union[torch.Tensor, List
     return out
 
 
+def permute_quantize(tokens: torch.Tensor, mappings: Union[torch.Tensor, List[int]]):
+    """``permute_tokens_cuda`` and the per-row fp8 quantisation in one kernel (no counterpart in the
+    reference, which has no fp8 path): ``(q [R, d] float8_e4m3fn, scale [R] fp32)`` with
+    ``q[mappings[t]] = fp8(tokens[t // k] / scale)``, ``scale = absmax / 448``.  Same bits as
+    ``quantize_rows(permute_tokens_cuda(tokens, mappings))``; the bf16 copy of the routed rows is never written."""
+    assert tokens.dim() == 2 and tokens.is_contiguous() and tokens.dtype in (torch.bfloat16, torch.float16)
+    device = _device_of(tokens)
+    tokens = tokens.to(device)
+    m = _index_tensor(mappings, device, torch.int64)
+    T, d = tokens.shape
+    R = m.numel()
+    assert T == 0 or R % T == 0, f"{R} mappings for {T} tokens"
+    q = torch.empty((R, d), dtype=torch.float8_e4m3fn, device=device)
+    scale = torch.empty(R, dtype=torch.float32, device=device)
+    with torch.cuda.device(device):
+        _lib.call("dmoe_permute_quant", tokens.data_ptr(), q.data_ptr(), scale.data_ptr(), m.data_ptr(),
+                  _INT_TYPES[m.dtype], T, R, d, _row_dtype(tokens), _stream(device))
+    return q, scale
+
+
 def permute_tokens_triton(tokens: torch.Tensor, mappings: Union[torch.Tensor, List[int]]) -> torch.Tensor:
     """Reference name kept (memory.py:72-91): the top-1 permute with int32 or
     int64 mappings.  Served by the same HIP kernel; there is no Triton here."""

@@ -200,6 +200,12 @@ int dmoe_gmm_tune(int variant);
 int dmoe_quant_rows(const void *x, void *q, float *scales, int64_t rows, int64_t d, int dtype,
                     void *stream);
 
+/* dmoe_permute followed by dmoe_quant_rows in one pass: q[mappings[t], :] = fp8(in[t / k, :] / s),
+ * scales[mappings[t]] = s = absmax(in[t / k, :]) / 448, k = R / T.  The token row is read once and stored k
+ * times as e4m3; the bf16 copy of the routed rows never exists.  Same bits as the two calls. */
+int dmoe_permute_quant(const void *in, void *q, float *scales, const void *mappings, int map_type, int64_t T,
+                       int64_t R, int64_t d, int dtype, void *stream);
+
 /* fp8 grouped GEMM, operands K-contiguous:
  *   a  fp8 [rows, K] with a_scale fp32 [rows]
  *   b  fp8 [E, N, K] with b_scale fp32 [E, N]     (per output channel)

@@ -154,3 +154,24 @@ def test_gmm_fp8_few_stages(variant, K):
         assert max_rel_err(out, exact) <= TOL_FP8
     finally:
         gg.set_tile_variant(0)
+
+
+@pytest.mark.parametrize("T,d,k,E", [(1, 16, 1, 1), (37, 1024, 2, 8), (100, 2048, 6, 64), (64, 6144, 2, 8), (5, 16384, 2, 4),
+                                     (3, 32768, 2, 2)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_permute_quantize_bit_exact(T, d, k, E, dtype):
+    # the fused kernel gives the bits of permute followed by quantise, and of the oracle's two steps
+    announce(test="permute_quantize", T=T, d=d, k=k, dtype=str(dtype))
+    from disagmoe_amd.ops import memory
+    from oracle import rows as orows, routing
+    g = torch.Generator().manual_seed(T * 7 + d)
+    x = (torch.randn(T, d, generator=g) * 3).to(dtype)
+    x[0, :] = 0 if T > 1 else x[0, :]                      # a zero row: scale 1
+    ids = torch.randint(0, E, (T * k,), generator=g)
+    m, _ = routing.get_mappings_from_exp_ids(ids, E)
+    q, s = memory.permute_quantize(x.to(dev()), torch.tensor(m, device=dev()))
+    q2, s2 = gg.quantize_rows(memory.permute_tokens_cuda(x.to(dev()), m))
+    assert torch.equal(q.view(torch.uint8), q2.view(torch.uint8)) and torch.equal(s, s2)
+    if dtype == torch.bfloat16:
+        q_ref, s_ref = fp8.quantize_rows(orows.permute_tokens(x, m))
+        assert torch.equal(q.cpu().view(torch.uint8), q_ref.view(torch.uint8)) and torch.equal(s.cpu(), s_ref)

@@ -175,3 +175,21 @@ def test_permute_quantize_bit_exact(T, d, k, E, dtype):
     if dtype == torch.bfloat16:
         q_ref, s_ref = fp8.quantize_rows(orows.permute_tokens(x, m))
         assert torch.equal(q.cpu().view(torch.uint8), q_ref.view(torch.uint8)) and torch.equal(s.cpu(), s_ref)
+
+
+def test_fp8_layer_fused_rows_equal_two_step():
+    # the layer quantises the routed rows on their way into the expert-sorted buffer; asking for the intermediate
+    # tensors takes the two-step path: the results have the same bits
+    announce(test="fp8_layer_fused_rows")
+    from disagmoe_amd.expert_layer import expert_layer_forward
+    E, d, I, T, k = 8, 1024, 1536, 300, 2
+    g = torch.Generator().manual_seed(17)
+    w13 = (torch.randn(E, d, 2 * I, generator=g) * 0.02).to(torch.bfloat16)
+    w2 = (torch.randn(E, I, d, generator=g) * 0.02).to(torch.bfloat16)
+    x = torch.randn(T, d, generator=g).to(torch.bfloat16).to(dev())
+    ids = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(dev())
+    gates = torch.softmax(torch.randn(T, k, generator=g), dim=-1).to(dev())
+    layer = MoEExpertsFP8(w13.to(dev()), w2.to(dev()))
+    fused = expert_layer_forward(layer, x, ids, gates)
+    two_step = expert_layer_forward(layer, x, ids, gates, stages={})
+    assert torch.equal(fused, two_step)

@@ -21,12 +21,16 @@ def _step(layer, x, logits, k):
     return expert_layer_forward(layer, x, ids, weights)
 
 
-@pytest.mark.parametrize("name,T", [("C1", 512), ("C3", 256), ("C4", 1024)])
-def test_graph_replays_equal_eager(name, T):
+@pytest.mark.parametrize("name,T,fp8", [("C1", 512, False), ("C3", 256, False), ("C4", 1024, False), ("C1", 512, True)])
+def test_graph_replays_equal_eager(name, T, fp8):
     w = workloads.WORKLOADS[name]
-    announce(test="graph_replay", config=name, T=T, d=w.d, I=w.I, E=w.E, k=w.k)
+    announce(test="graph_replay", config=name, T=T, d=w.d, I=w.I, E=w.E, k=w.k, fp8=fp8)
     w13, w2 = workloads.make_weights(w, dev())
-    layer = _layer_from(w13, w2)
+    if fp8:   # the fp8 step: rows quantised inside the permute, the intermediate quantised between the GEMMs
+        from disagmoe_amd.models.experts import MoEExpertsFP8
+        layer = MoEExpertsFP8(w13, w2)
+    else:
+        layer = _layer_from(w13, w2)
     g = torch.Generator().manual_seed(77)
     x_static = torch.zeros(T, w.d, dtype=torch.bfloat16, device=dev())
     logits_static = torch.zeros(T, w.E, dtype=torch.float32, device=dev())

@@ -41,12 +41,16 @@ def _tile_rows(w) -> int:
     return tile
 
 
-def _event_ms(fn, iters: int, warmup: int = 2):
+def _event_ms(fn, iters: int, warmup: int = 2, plug=None):
     """Average duration of ``fn`` in ms, HIP events on the current stream (the one
-    the kernels are launched on)."""
+    the kernels are launched on).  ``plug`` is device work of a few ms enqueued first:
+    the events and launches of a kernel that is shorter than its own host call then
+    queue up behind it and the intervals hold no time spent waiting for the host."""
     import torch
     for _ in range(warmup):
         fn()
+    if plug is not None:
+        plug()
     start = [torch.cuda.Event(enable_timing=True) for _ in range(iters)]
     stop = [torch.cuda.Event(enable_timing=True) for _ in range(iters)]
     for i in range(iters):
@@ -171,10 +175,31 @@ def main() -> int:
     permuted = memory.permute_tokens_cuda(x, mappings)
     it = args.kernel_iters
     stages = {}
-    ms, _ = _event_ms(lambda: memory.route_tokens(ids, w.E), it)
+    # the row kernels take 5 - 100 us, less than the host needs to launch them from Python
+    plug_a = torch.randn(8192, 8192, dtype=torch.bfloat16, device=dev)
+    plug_c = torch.empty_like(plug_a)
+
+    def plug():
+        for _ in range(4):
+            torch.mm(plug_a, plug_a, out=plug_c)
+
+    ms, _ = _event_ms(lambda: memory.route_tokens(ids, w.E), it, plug=plug)
     stages["route"] = {"ms": ms, "GB/s": w.route_bytes / ms / 1e6}
-    ms, _ = _event_ms(lambda: memory.permute_tokens_cuda(x, mappings), it)
-    stages["permute"] = {"ms": ms, "GB/s": w.permute_bytes / ms / 1e6, "frac_hbm": w.permute_bytes / ms / 1e6 / PEAK_HBM_GBS}
+    def sustained_ms(fn, n=10):
+        """ms per launch when n launches follow each other inside one event interval: a launch's ramp-up overlaps the
+        drain of the one before it, as it does behind another kernel in a running step"""
+        def many():
+            for _ in range(n):
+                fn()
+        return _event_ms(many, max(2, it // 2), plug=plug)[0] / n
+
+    ms, _ = _event_ms(lambda: memory.permute_tokens_cuda(x, mappings), it, plug=plug)
+    # "GB/s" counts a read and a write per routed row; the kernel reads a token once for its k copies ("moved")
+    moved = (w.T + w.R) * w.d * 2 + 8.0 * w.R
+    stages["permute"] = {"ms": ms, "GB/s": w.permute_bytes / ms / 1e6, "frac_hbm": w.permute_bytes / ms / 1e6 / PEAK_HBM_GBS,
+                         "GB/s_moved": moved / ms / 1e6, "frac_hbm_moved": moved / ms / 1e6 / PEAK_HBM_GBS}
+    ms = sustained_ms(lambda: memory.permute_tokens_cuda(x, mappings))
+    stages["permute"].update({"ms_back_to_back": ms, "frac_hbm_back_to_back": w.permute_bytes / ms / 1e6 / PEAK_HBM_GBS})
     if w.fp8:
         xq, xs = gg.quantize_rows(permuted)
         h = gg.gmm_fp8_swiglu(xq, xs, layer.w13_q, layer.w13_scale, batch_sizes)
@@ -207,8 +232,10 @@ def main() -> int:
     stages["gemm_total"] = {"ms": up_ms + down_ms, "TFLOP/s": w.gemm_flops / (up_ms + down_ms) / 1e9,
                             "frac_mfma": w.gemm_flops / (up_ms + down_ms) / 1e9 / peak}
     y = layer.forward(w.R, permuted, batch_sizes)
-    ms, _ = _event_ms(lambda: memory.combine_tokens(y, mappings, gates), it)
+    ms, _ = _event_ms(lambda: memory.combine_tokens(y, mappings, gates), it, plug=plug)
     stages["combine"] = {"ms": ms, "GB/s": w.combine_bytes / ms / 1e6, "frac_hbm": w.combine_bytes / ms / 1e6 / PEAK_HBM_GBS}
+    ms = sustained_ms(lambda: memory.combine_tokens(y, mappings, gates))
+    stages["combine"].update({"ms_back_to_back": ms, "frac_hbm_back_to_back": w.combine_bytes / ms / 1e6 / PEAK_HBM_GBS})
 
     achieved = up_flops / up_ms / 1e9
     roofline = {"kernel": kernel, "bound": "mfma", "achieved": achieved, "peak": peak, "unit": "TFLOP/s",

@@ -51,11 +51,28 @@ bool first_on_device(unsigned long long *seen) {
 constexpr int kChunk = 512;       // rows per wavefront
 constexpr int kMaxExperts = 4096; // 3 int tables of E entries must fit in LDS
 
+// The ids of rows base + i * 64 + lane, i < kChunk / 64, of a chunk: -2 past the end, -1 present but outside
+// [0, E).  Every load is issued before the first value is looked at (rows past the end re-read the last row).
 template <typename IdT>
-__device__ __forceinline__ int load_id(const IdT *ids, int64_t t, int64_t R, int E) {
-    if (t >= R) return -2;  // past the end
-    long long v = (long long)ids[t];
-    return (v >= 0 && v < E) ? (int)v : -1;  // -1: present but invalid
+__device__ __forceinline__ void load_chunk_ids(const IdT *ids, int64_t base, int lane, int64_t R, int E,
+                                               int (&out)[kChunk / kWave]) {
+    IdT raw[kChunk / kWave];
+    if (R <= 0) {   // no row to re-read (and ids may be null)
+#pragma unroll
+        for (int i = 0; i < kChunk / kWave; ++i) out[i] = -2;
+        return;
+    }
+#pragma unroll
+    for (int i = 0; i < kChunk / kWave; ++i) {
+        const int64_t t = base + i * kWave + lane;
+        raw[i] = ids[t < R ? t : R - 1];
+    }
+#pragma unroll
+    for (int i = 0; i < kChunk / kWave; ++i) {
+        const int64_t t = base + i * kWave + lane;
+        const long long v = (long long)raw[i];
+        out[i] = t >= R ? -2 : ((v >= 0 && v < E) ? (int)v : -1);
+    }
 }
 
 template <typename IdT>
@@ -66,10 +83,11 @@ __global__ __launch_bounds__(kWave) void route_hist_kernel(const IdT *__restrict
     const int64_t base = (int64_t)blockIdx.x * kChunk;
     for (int e = lane; e < E; e += kWave) cnt[e] = 0;
     __syncthreads();
-    for (int i = 0; i < kChunk; i += kWave) {
-        int id = load_id(ids, base + i + lane, R, E);
-        if (id >= 0) atomicAdd(&cnt[id], 1);
-    }
+    int my_id[kChunk / kWave];
+    load_chunk_ids(ids, base, lane, R, E, my_id);
+#pragma unroll
+    for (int i = 0; i < kChunk / kWave; ++i)
+        if (my_id[i] >= 0) atomicAdd(&cnt[my_id[i]], 1);
     __syncthreads();
     for (int e = lane; e < E; e += kWave) chunk_hist[(int64_t)blockIdx.x * E + e] = cnt[e];
 }
@@ -88,23 +106,51 @@ __global__ __launch_bounds__(kWave) void route_map_kernel(const IdT *__restrict_
     const int chunk = blockIdx.x;
     const int64_t base = (int64_t)chunk * kChunk;
 
+    // this lane's rows of the chunk, all loads in flight before anything waits for one
+    constexpr int kPerLane = kChunk / kWave;
+    int my_id[kPerLane];
+    load_chunk_ids(ids, base, lane, R, E, my_id);
+
     if (kSingle) {
         for (int e = lane; e < E; e += kWave) { tot[e] = 0; run[e] = 0; }
         __syncthreads();
-        for (int i = 0; i < kChunk; i += kWave) {
-            int id = load_id(ids, base + i + lane, R, E);
-            if (id >= 0) atomicAdd(&tot[id], 1);
-        }
+#pragma unroll
+        for (int i = 0; i < kPerLane; ++i)
+            if (my_id[i] >= 0) atomicAdd(&tot[my_id[i]], 1);
     } else {
-        for (int e = lane; e < E; e += kWave) {
+        // Column sums of chunk_hist[nchunks][E]: all rows (tot) and the rows before this chunk (run).  A lane owns
+        // expert e0 + lane % span and every slices-th row from row lane / span on, kBatch loads in flight at a
+        // time; the slices are added up across the wavefront.
+        constexpr int kBatch = 16;
+        int span = kWave;
+        while (span / 2 >= E) span /= 2;   // lanes per slice: the power of two that covers E, at most a wavefront
+        const int slices = kWave / span, slice = lane / span, el = lane % span;
+        for (int e0 = 0; e0 < E; e0 += span) {
+            const int e = e0 + el;
             int before = 0, all = 0;
-            for (int c = 0; c < nchunks; ++c) {
-                int v = chunk_hist[(int64_t)c * E + e];
-                all += v;
-                if (c < chunk) before += v;
+            if (e < E) {
+                for (int c0 = slice; c0 < nchunks; c0 += slices * kBatch) {
+                    int v[kBatch];
+#pragma unroll
+                    for (int u = 0; u < kBatch; ++u) {
+                        const int c = c0 + u * slices;
+                        v[u] = c < nchunks ? chunk_hist[(int64_t)c * E + e] : 0;
+                    }
+#pragma unroll
+                    for (int u = 0; u < kBatch; ++u) {
+                        all += v[u];
+                        if (c0 + u * slices < chunk) before += v[u];
+                    }
+                }
             }
-            run[e] = before;
-            tot[e] = all;
+            for (int s = span; s < kWave; s <<= 1) {
+                before += __shfl_xor(before, s, kWave);
+                all += __shfl_xor(all, s, kWave);
+            }
+            if (e < E && slice == 0) {
+                run[e] = before;
+                tot[e] = all;
+            }
         }
     }
     __syncthreads();
@@ -137,9 +183,10 @@ __global__ __launch_bounds__(kWave) void route_map_kernel(const IdT *__restrict_
     while ((1 << nbits) < E) ++nbits;
     const unsigned long long below = (lane == 0) ? 0ull : (~0ull >> (kWave - lane));
 
-    for (int i = 0; i < kChunk; i += kWave) {
-        const int64_t t = base + i + lane;
-        const int id = load_id(ids, t, R, E);
+#pragma unroll
+    for (int i = 0; i < kPerLane; ++i) {
+        const int64_t t = base + i * kWave + lane;
+        const int id = my_id[i];
         const bool ok = id >= 0;
         unsigned long long same = __ballot(ok);
         for (int b = 0; b < nbits; ++b) {

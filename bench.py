@@ -199,7 +199,7 @@ def main() -> int:
     stages["permute"] = {"ms": ms, "GB/s": w.permute_bytes / ms / 1e6, "frac_hbm": w.permute_bytes / ms / 1e6 / PEAK_HBM_GBS,
                          "GB/s_moved": moved / ms / 1e6, "frac_hbm_moved": moved / ms / 1e6 / PEAK_HBM_GBS}
     ms = sustained_ms(lambda: memory.permute_tokens_cuda(x, mappings))
-    stages["permute"].update({"ms_back_to_back": ms, "frac_hbm_back_to_back": w.permute_bytes / ms / 1e6 / PEAK_HBM_GBS})
+    stages["permute"].update({"ms_back_to_back": ms, "frac_hbm_moved_back_to_back": moved / ms / 1e6 / PEAK_HBM_GBS})
     if w.fp8:
         xq, xs = gg.quantize_rows(permuted)
         h = gg.gmm_fp8_swiglu(xq, xs, layer.w13_q, layer.w13_scale, batch_sizes)

@@ -8,7 +8,12 @@
 //           expert) and all of them (counts, offsets), then walks its rows 64 at a
 //           time; a row's rank inside the 64 is the number of lower lanes with
 //           the same id, found with log2(E) wave ballots.
-// With a single chunk the two passes run in one launch.
+// Up to 12 chunks run both passes in one launch of one workgroup, a wavefront
+// per chunk and the histograms in LDS.  When summing the
+// histograms would take a wavefront of pass 2 more than two batches of loads, a
+// launch between the two turns them into their running sums over the chunks and
+// pass 2 reads one row instead of all rows (its work would grow with the square
+// of the chunk count).
 #include <stdarg.h>
 #include <string.h>
 
@@ -50,6 +55,11 @@ bool first_on_device(unsigned long long *seen) {
 
 constexpr int kChunk = 512;       // rows per wavefront
 constexpr int kMaxExperts = 4096; // 3 int tables of E entries must fit in LDS
+// chunks that one workgroup takes, a wavefront each, when their tables fit in LDS (measured: 6144 rows 13 us against
+// 16 us for two launches, 8192 rows 16 us against 15 us)
+constexpr int kBlockChunks = 12;
+constexpr int kSumBatch = 16;     // histogram rows a lane of pass 2 has in flight
+constexpr int kScanWaves = 16;    // wavefronts of a scanning workgroup
 
 // The ids of rows base + i * 64 + lane, i < kChunk / 64, of a chunk: -2 past the end, -1 present but outside
 // [0, E).  Every load is issued before the first value is looked at (rows past the end re-read the last row).
@@ -92,18 +102,68 @@ __global__ __launch_bounds__(kWave) void route_hist_kernel(const IdT *__restrict
     for (int e = lane; e < E; e += kWave) chunk_hist[(int64_t)blockIdx.x * E + e] = cnt[e];
 }
 
-template <typename IdT, typename MapT, bool kSingle>
-__global__ __launch_bounds__(kWave) void route_map_kernel(const IdT *__restrict__ ids, int64_t R, int E, int nchunks,
-                                                         const int *__restrict__ chunk_hist, int order,
+// chunk_hist[nchunks][E] -> exclusive running sums over the chunks, in place, and totals[E].  A workgroup owns 64
+// experts (lane = expert: rows of the table are read 256 bytes at a time), each of its wavefronts a contiguous range
+// of chunks: sum of the range, offsets of the ranges through LDS, then the range again, a batch of loads at a time.
+__global__ __launch_bounds__(kScanWaves *kWave) void route_scan_kernel(int *__restrict__ chunk_hist, int nchunks, int E,
+                                                                      int *__restrict__ totals) {
+    __shared__ int part[kScanWaves][kWave];
+    constexpr int kBatch = 16;
+    const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+    const int e = blockIdx.x * kWave + lane;
+    const int per = (nchunks + kScanWaves - 1) / kScanWaves;
+    const int c_lo = wave * per < nchunks ? wave * per : nchunks;
+    const int c_hi = c_lo + per < nchunks ? c_lo + per : nchunks;
+    int sum = 0;
+    if (e < E) {
+        for (int c0 = c_lo; c0 < c_hi; c0 += kBatch) {
+            int v[kBatch];
+#pragma unroll
+            for (int u = 0; u < kBatch; ++u) v[u] = c0 + u < c_hi ? chunk_hist[(int64_t)(c0 + u) * E + e] : 0;
+#pragma unroll
+            for (int u = 0; u < kBatch; ++u) sum += v[u];
+        }
+    }
+    part[wave][lane] = sum;
+    __syncthreads();
+    int run = 0, all = 0;
+#pragma unroll
+    for (int w = 0; w < kScanWaves; ++w) {
+        const int v = part[w][lane];
+        if (w < wave) run += v;
+        all += v;
+    }
+    if (e >= E) return;
+    if (wave == 0) totals[e] = all;
+    for (int c0 = c_lo; c0 < c_hi; c0 += kBatch) {
+        int v[kBatch];
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) v[u] = c0 + u < c_hi ? chunk_hist[(int64_t)(c0 + u) * E + e] : 0;
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) {
+            if (c0 + u < c_hi) chunk_hist[(int64_t)(c0 + u) * E + e] = run;
+            run += v[u];
+        }
+    }
+}
+
+// kMode 0: a workgroup (one wavefront) per chunk, chunk_hist holds the histograms of all chunks; 2: the same, but
+// chunk_hist holds the running sums over the chunks (route_scan_kernel) and `totals` the column sums; 1: the whole
+// problem in one workgroup, a wavefront per chunk, histograms and their running sums in LDS, no chunk_hist.
+template <typename IdT, typename MapT, int kMode>
+__global__ __launch_bounds__(kMode == 1 ? kBlockChunks * kWave : kWave) void route_map_kernel(const IdT *__restrict__ ids, int64_t R, int E, int nchunks,
+                                                         const int *__restrict__ chunk_hist,
+                                                         const int *__restrict__ totals, int order,
                                                          MapT *__restrict__ mappings,
                                                          int64_t *__restrict__ batch_sizes,
                                                          int64_t *__restrict__ offsets) {
     extern __shared__ int sm[];
-    int *run = sm;           // rows of expert e seen before the current 64
-    int *excl = sm + E;      // first destination row of expert e
-    int *tot = sm + 2 * E;   // rows of expert e
-    const int lane = threadIdx.x;
-    const int chunk = blockIdx.x;
+    constexpr bool kSingle = kMode == 1;
+    const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+    const int chunk = kSingle ? wave : blockIdx.x;
+    int *excl = sm;                                    // first destination row of expert e
+    int *tot = sm + E;                                 // rows of expert e
+    int *run = sm + 2 * E + (kSingle ? wave * E : 0);  // rows of expert e before the current 64 (a table per chunk)
     const int64_t base = (int64_t)chunk * kChunk;
 
     // this lane's rows of the chunk, all loads in flight before anything waits for one
@@ -111,17 +171,34 @@ __global__ __launch_bounds__(kWave) void route_map_kernel(const IdT *__restrict_
     int my_id[kPerLane];
     load_chunk_ids(ids, base, lane, R, E, my_id);
 
-    if (kSingle) {
-        for (int e = lane; e < E; e += kWave) { tot[e] = 0; run[e] = 0; }
+    if (kMode == 2) {
+        for (int e = lane; e < E; e += kWave) {
+            run[e] = chunk_hist[(int64_t)chunk * E + e];
+            tot[e] = totals[e];
+        }
+    } else if (kSingle) {
+        const int nw = blockDim.x / kWave;
+        for (int e = lane; e < E; e += kWave) run[e] = 0;
         __syncthreads();
 #pragma unroll
         for (int i = 0; i < kPerLane; ++i)
-            if (my_id[i] >= 0) atomicAdd(&tot[my_id[i]], 1);
+            if (my_id[i] >= 0) atomicAdd(&run[my_id[i]], 1);
+        __syncthreads();
+        // histogram of chunk w -> rows of the chunks before w, and the column sums
+        for (int e = threadIdx.x; e < E; e += blockDim.x) {
+            int acc = 0;
+            for (int w = 0; w < nw; ++w) {
+                const int v = sm[(2 + w) * E + e];
+                sm[(2 + w) * E + e] = acc;
+                acc += v;
+            }
+            tot[e] = acc;
+        }
     } else {
         // Column sums of chunk_hist[nchunks][E]: all rows (tot) and the rows before this chunk (run).  A lane owns
         // expert e0 + lane % span and every slices-th row from row lane / span on, kBatch loads in flight at a
         // time; the slices are added up across the wavefront.
-        constexpr int kBatch = 16;
+        constexpr int kBatch = kSumBatch;
         int span = kWave;
         while (span / 2 >= E) span /= 2;   // lanes per slice: the power of two that covers E, at most a wavefront
         const int slices = kWave / span, slice = lane / span, el = lane % span;
@@ -166,7 +243,7 @@ __global__ __launch_bounds__(kWave) void route_map_kernel(const IdT *__restrict_
             int up = __shfl_up(incl, s, kWave);
             if (lane >= s) incl += up;
         }
-        if (e < E) excl[e] = carry + incl - v;
+        if (e < E && wave == 0) excl[e] = carry + incl - v;
         carry += __shfl(incl, kWave - 1, kWave);
     }
     __syncthreads();
@@ -210,23 +287,43 @@ __global__ __launch_bounds__(kWave) void route_map_kernel(const IdT *__restrict_
     }
 }
 
+// a few chunks are routed by a single workgroup if its 2 + nchunks tables fit in 64 KiB of LDS
+static bool one_workgroup(int64_t nchunks, int E) {
+    return nchunks <= 1 || (nchunks <= kBlockChunks && (2 + nchunks) * (int64_t)E * (int64_t)sizeof(int) <= (64 << 10));
+}
+
 template <typename IdT, typename MapT>
 static int launch_route(const void *ids, int64_t R, int E, int order, void *mappings, int64_t *batch_sizes,
                         int64_t *offsets, void *scratch, hipStream_t stream) {
     const int nchunks = (int)((R + kChunk - 1) / kChunk);
     const size_t lds = 3 * (size_t)E * sizeof(int);
-    if (nchunks <= 1) {
-        hipLaunchKernelGGL((route_map_kernel<IdT, MapT, true>), dim3(1), dim3(kWave), lds, stream, (const IdT *)ids, R,
-                           E, 1, (const int *)nullptr, order, (MapT *)mappings, batch_sizes, offsets);
+    if (one_workgroup(nchunks, E)) {
+        const int nw = nchunks < 1 ? 1 : nchunks;
+        hipLaunchKernelGGL((route_map_kernel<IdT, MapT, 1>), dim3(1), dim3(nw * kWave), (2 + nw) * (size_t)E * sizeof(int),
+                           stream, (const IdT *)ids, R, E, nw, (const int *)nullptr, (const int *)nullptr, order,
+                           (MapT *)mappings, batch_sizes, offsets);
         DMOE_LAUNCH_CHECK("route_map_kernel");
         return DMOE_OK;
     }
+    int *hist = (int *)scratch;
     hipLaunchKernelGGL((route_hist_kernel<IdT>), dim3(nchunks), dim3(kWave), (size_t)E * sizeof(int), stream,
-                       (const IdT *)ids, R, E, (int *)scratch);
+                       (const IdT *)ids, R, E, hist);
     DMOE_LAUNCH_CHECK("route_hist_kernel");
-    hipLaunchKernelGGL((route_map_kernel<IdT, MapT, false>), dim3(nchunks), dim3(kWave), lds, stream,
-                       (const IdT *)ids, R, E, nchunks, (const int *)scratch, order, (MapT *)mappings, batch_sizes,
-                       offsets);
+    int span = kWave;   // lanes of pass 2 that share a histogram row (see route_map_kernel)
+    while (span / 2 >= E) span /= 2;
+    if (nchunks > 2 * kSumBatch * (kWave / span)) {
+        int *totals = hist + (size_t)nchunks * E;
+        hipLaunchKernelGGL(route_scan_kernel, dim3((E + kWave - 1) / kWave), dim3(kScanWaves * kWave), 0, stream, hist,
+                           nchunks, E, totals);
+        DMOE_LAUNCH_CHECK("route_scan_kernel");
+        hipLaunchKernelGGL((route_map_kernel<IdT, MapT, 2>), dim3(nchunks), dim3(kWave), lds, stream, (const IdT *)ids,
+                           R, E, nchunks, (const int *)hist, (const int *)totals, order, (MapT *)mappings, batch_sizes,
+                           offsets);
+    } else {
+        hipLaunchKernelGGL((route_map_kernel<IdT, MapT, 0>), dim3(nchunks), dim3(kWave), lds, stream, (const IdT *)ids,
+                           R, E, nchunks, (const int *)hist, (const int *)nullptr, order, (MapT *)mappings, batch_sizes,
+                           offsets);
+    }
     DMOE_LAUNCH_CHECK("route_map_kernel");
     return DMOE_OK;
 }
@@ -249,7 +346,8 @@ extern "C" int dmoe_route_scratch_bytes(int64_t R, int E, size_t *bytes) {
     DMOE_REQUIRE(R >= 0 && R < (1ll << 31), DMOE_ERR_SHAPE, "dmoe_route: R=%lld outside [0, 2^31)", (long long)R);
     DMOE_REQUIRE(E > 0 && E <= kMaxExperts, DMOE_ERR_SHAPE, "dmoe_route: E=%d outside [1, %d]", E, kMaxExperts);
     const int64_t nchunks = (R + kChunk - 1) / kChunk;
-    *bytes = (nchunks <= 1) ? 0 : (size_t)nchunks * (size_t)E * sizeof(int);
+    // a histogram per chunk and, behind them, the column sums of the scanned form
+    *bytes = one_workgroup(nchunks, E) ? 0 : (size_t)(nchunks + 1) * (size_t)E * sizeof(int);
     return DMOE_OK;
 }
 

@@ -42,7 +42,7 @@ def test_known_answers(golden_dir):
         assert empty == [] and m32.dtype == torch.int32 and m32.cpu().tolist() == case["stable"]
 
 
-@pytest.mark.parametrize("R", [1, 63, 64, 65, 511, 512, 513, 1024, 5000, 49152])
+@pytest.mark.parametrize("R", [1, 63, 64, 65, 511, 512, 513, 1024, 5000, 6144, 6145, 16384, 16385, 16897, 49152, 300007])
 @pytest.mark.parametrize("E", [1, 2, 8, 64, 100])
 def test_random_ids(R, E):
     announce(test="route_random", R=R, E=E)
@@ -108,5 +108,8 @@ def test_expert_count_limits():
     g = torch.Generator().manual_seed(11)
     _check(torch.randint(0, 4096, (10000,), generator=g), 4096)
     _check(torch.randint(4000, 4096, (300,), generator=g), 4096)      # one chunk, nearly all experts empty
+    _check(torch.randint(0, 4096, (40000,), generator=g), 4096)       # scanned histograms, 64 workgroups of experts
+    _check(torch.randint(0, 4096, (1000,), generator=g), 4096)        # two chunks in one workgroup: 64 KiB of LDS
+    _check(torch.randint(0, 4096, (1500,), generator=g), 4096)        # three chunks: their tables no longer fit
     with pytest.raises(DmoeError):
         memory.route_tokens(torch.zeros(8, dtype=torch.int64, device=dev()), 4097)

@@ -26,7 +26,7 @@ PEAK_FP8_TFLOPS = 5000.0
 
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc runs (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0,
 # the factors read off a 1 GiB copy in the same runs: profiles/expert_layer_c2_hbm_traffic.md); None = not measured.
-MEASURED_TRAFFIC = {"C2": 6.11e9}
+MEASURED_TRAFFIC = {"C2": 6.11e9, "C4": 1.551e9, "C5": 13.95e9}
 
 
 def _tile_rows(w) -> int:

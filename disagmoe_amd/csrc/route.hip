@@ -105,10 +105,10 @@ __global__ __launch_bounds__(kWave) void route_hist_kernel(const IdT *__restrict
 // chunk_hist[nchunks][E] -> exclusive running sums over the chunks, in place, and totals[E].  A workgroup owns 64
 // experts (lane = expert: rows of the table are read 256 bytes at a time), each of its wavefronts a contiguous range
 // of chunks: sum of the range, offsets of the ranges through LDS, then the range again, a batch of loads at a time.
-__global__ __launch_bounds__(kScanWaves *kWave) void route_scan_kernel(int *__restrict__ chunk_hist, int nchunks, int E,
-                                                                      int *__restrict__ totals) {
+__global__ __launch_bounds__(kScanWaves * kWave) void route_scan_kernel(int *__restrict__ chunk_hist, int nchunks, int E,
+                                                                       int *__restrict__ totals) {
     __shared__ int part[kScanWaves][kWave];
-    constexpr int kBatch = 16;
+    constexpr int kBatch = kSumBatch;
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
     const int e = blockIdx.x * kWave + lane;
     const int per = (nchunks + kScanWaves - 1) / kScanWaves;
@@ -151,12 +151,10 @@ __global__ __launch_bounds__(kScanWaves *kWave) void route_scan_kernel(int *__re
 // chunk_hist holds the running sums over the chunks (route_scan_kernel) and `totals` the column sums; 1: the whole
 // problem in one workgroup, a wavefront per chunk, histograms and their running sums in LDS, no chunk_hist.
 template <typename IdT, typename MapT, int kMode>
-__global__ __launch_bounds__(kMode == 1 ? kBlockChunks * kWave : kWave) void route_map_kernel(const IdT *__restrict__ ids, int64_t R, int E, int nchunks,
-                                                         const int *__restrict__ chunk_hist,
-                                                         const int *__restrict__ totals, int order,
-                                                         MapT *__restrict__ mappings,
-                                                         int64_t *__restrict__ batch_sizes,
-                                                         int64_t *__restrict__ offsets) {
+__global__ __launch_bounds__(kMode == 1 ? kBlockChunks * kWave : kWave) void route_map_kernel(
+    const IdT *__restrict__ ids, int64_t R, int E, int nchunks, const int *__restrict__ chunk_hist,
+    const int *__restrict__ totals, int order, MapT *__restrict__ mappings, int64_t *__restrict__ batch_sizes,
+    int64_t *__restrict__ offsets) {
     extern __shared__ int sm[];
     constexpr bool kSingle = kMode == 1;
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;

@@ -1,8 +1,9 @@
 // Routing producer: softmax over the router logits of a token, its k largest probabilities and
 // their expert ids, optionally renormalised to sum 1.
 //
-// A token is handled by a group of W lanes (W = 8, 16, 32 or 64, the power of two that covers E,
-// 64 beyond that), 64 / W tokens per wavefront; a lane keeps ceil(E / W) logits in registers.
+// A token is handled by a group of W lanes (W = 8, 16, 32 or 64), 64 / W tokens per wavefront; a lane
+// keeps ceil(E / W) logits in registers.  Few tokens: W is the power of two that covers E (64 beyond
+// that); many tokens: W = 8 or 16 with up to 16 logits per lane.
 // Max, sum and the k arg-max rounds are butterfly reductions inside the group; every lane of the
 // group ends up with the same winner, so there is no LDS and no atomics.  Ties go to the lower
 // expert id.  The work is one read of the logits: HBM-bound, a few microseconds at serving sizes.
@@ -107,11 +108,24 @@ static int launch_topk(const void *logits, int64_t n, int E, int k, int renormal
 template <typename T, typename IdT>
 static int launch_topk_by_width(const void *logits, int64_t n, int E, int k, int renormalize, float *weights,
                                 void *ids, hipStream_t stream) {
+    // A round of the arg-max costs a lane VPL compares and log2(W) exchanges, and a token W lanes of that: narrow
+    // groups do less work in all, wide groups have the shorter chain of dependent instructions.  Few tokens (every
+    // wavefront of the wide form resident at once, two per SIMD at most) are latency-bound and take the wide form
+    // (512 tokens x 64 experts: 8 against 10 us), many take the narrow one (8192 x 64: 13 against 20 us).
+    const bool few = n * (E <= 8 ? 8 : E <= 16 ? 16 : E <= 32 ? 32 : 64) / kWave <= 2048;
     if (E <= 8) return launch_topk<T, IdT, 8, 1>(logits, n, E, k, renormalize, weights, ids, stream);
-    if (E <= 16) return launch_topk<T, IdT, 16, 1>(logits, n, E, k, renormalize, weights, ids, stream);
-    if (E <= 32) return launch_topk<T, IdT, 32, 1>(logits, n, E, k, renormalize, weights, ids, stream);
-    if (E <= 64) return launch_topk<T, IdT, 64, 1>(logits, n, E, k, renormalize, weights, ids, stream);
-    if (E <= 256) return launch_topk<T, IdT, 64, 4>(logits, n, E, k, renormalize, weights, ids, stream);
+    if (few) {
+        if (E <= 16) return launch_topk<T, IdT, 16, 1>(logits, n, E, k, renormalize, weights, ids, stream);
+        if (E <= 32) return launch_topk<T, IdT, 32, 1>(logits, n, E, k, renormalize, weights, ids, stream);
+        if (E <= 64) return launch_topk<T, IdT, 64, 1>(logits, n, E, k, renormalize, weights, ids, stream);
+        if (E <= 256) return launch_topk<T, IdT, 64, 4>(logits, n, E, k, renormalize, weights, ids, stream);
+    } else {
+        if (E <= 16) return launch_topk<T, IdT, 8, 2>(logits, n, E, k, renormalize, weights, ids, stream);
+        if (E <= 32) return launch_topk<T, IdT, 8, 4>(logits, n, E, k, renormalize, weights, ids, stream);
+        if (E <= 64) return launch_topk<T, IdT, 8, 8>(logits, n, E, k, renormalize, weights, ids, stream);
+        if (E <= 128) return launch_topk<T, IdT, 16, 8>(logits, n, E, k, renormalize, weights, ids, stream);
+        if (E <= 256) return launch_topk<T, IdT, 16, 16>(logits, n, E, k, renormalize, weights, ids, stream);
+    }
     return launch_topk<T, IdT, 64, 16>(logits, n, E, k, renormalize, weights, ids, stream);
 }
 

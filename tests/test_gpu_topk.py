@@ -25,7 +25,10 @@ def _check(x_cpu: torch.Tensor, k: int, renorm: bool, ids_dtype=torch.int32):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("n,E,k", [(1, 8, 2), (4096, 8, 2), (8192, 64, 6), (257, 5, 5), (100, 16, 1), (63, 32, 4),
-                                   (300, 160, 8), (77, 1000, 32), (50, 256, 3), (31, 65, 7)])
+                                   (300, 160, 8), (77, 1000, 32), (50, 256, 3), (31, 65, 7),
+                                   # many tokens: narrow lane groups with several logits per lane
+                                   (20000, 16, 2), (10000, 32, 4), (3000, 100, 8), (2500, 160, 6), (2100, 256, 32),
+                                   (2049, 65, 7)])
 def test_fused_topk(n, E, k, dtype):
     announce(test="fused_topk", n=n, E=E, k=k, dtype=str(dtype))
     g = torch.Generator().manual_seed(n * 131 + E)
@@ -39,6 +42,8 @@ def test_ties_and_masked_experts():
     x = torch.tensor([[1, 5, 5, 0, 5, 5, 5, 5], [0, 0, 0, 0, 0, 0, 0, 0]], dtype=torch.float32)
     _check(x, 3, True)
     x = torch.randint(-2, 3, (500, 12), generator=torch.Generator().manual_seed(3)).float()
+    _check(x, 4, True)
+    x = torch.randint(-2, 3, (10000, 12), generator=torch.Generator().manual_seed(5)).float()   # the narrow form
     _check(x, 4, True)
     x = torch.randn(64, 16, generator=torch.Generator().manual_seed(4))
     x[:, ::3] = float("-inf")                   # masked experts: probability 0, never ahead of a finite logit

@@ -50,7 +50,7 @@ __device__ __forceinline__ u32x4 scale_f16x8(u32x4 v, float s) {
 }
 
 // out[map[i*k + j]] = in[i] (* scale[i*k + j]); one wavefront per (token i, segment).
-template <typename MapT, int kScale /*0 none, 1 bf16, 2 fp16*/>
+template <typename MapT, int kScale /*0 none, 1 bf16, 2 fp16*/, bool kStreamed>
 __global__ __launch_bounds__(kBlock) void permute_kernel(const u32x4 *__restrict__ in, u32x4 *__restrict__ out,
                                                         const MapT *__restrict__ map, int64_t T, int k, int64_t R,
                                                         int vecs, int nseg, const uint16_t *__restrict__ scale) {
@@ -82,7 +82,9 @@ __global__ __launch_bounds__(kBlock) void permute_kernel(const u32x4 *__restrict
                 u32x4 x = buf[u];
                 if (kScale == 1) x = scale_bf16x8(x, s);
                 if (kScale == 2) x = scale_f16x8(x, s);
-                dst[v] = x;
+                // an output larger than the last-level cache is written past it
+                if (kStreamed) __builtin_nontemporal_store(x, dst + v);
+                else dst[v] = x;
             }
         }
     }
@@ -196,7 +198,7 @@ __global__ __launch_bounds__(kBlock) void combine_kernel(const u32x4 *__restrict
 // q[map[i*k + j], :] = fp8(x[i, :] / s[i]) and scales[map[i*k + j]] = s[i] for j < k: the permute and the per-row
 // quantisation in one pass (without a mapping: the quantisation alone, q[i, :] and scales[i]).  One workgroup per token;
 // the row is read once (kept in registers when it has at most 16384 elements), quantised once and stored k times.
-template <typename MapT, bool kHalf>
+template <typename MapT, bool kHalf, bool kStreamed>
 __global__ __launch_bounds__(kBlock) void permute_quant_kernel(const u32x4 *__restrict__ x, uint2 *__restrict__ q,
                                                               float *__restrict__ scales, const MapT *__restrict__ map,
                                                               int k, int64_t R, int vecs) {
@@ -257,7 +259,10 @@ __global__ __launch_bounds__(kBlock) void permute_quant_kernel(const u32x4 *__re
 #pragma unroll
             for (int u = 0; u < kKeep; ++u) {
                 const int v = threadIdx.x + u * kBlock;
-                if (v < vecs) dst[v] = out[u];
+                if (v >= vecs) continue;
+                if (kStreamed)
+                    __builtin_nontemporal_store(((unsigned long long)out[u].y << 32) | out[u].x, (unsigned long long *)(dst + v));
+                else dst[v] = out[u];
             }
         }
     } else {
@@ -308,9 +313,17 @@ extern "C" int dmoe_permute(const void *in, void *out, const void *mappings, int
     DMOE_REQUIRE(nblk < (1ll << 31), DMOE_ERR_SHAPE, "dmoe_permute: too many rows");
     hipStream_t s = (hipStream_t)stream;
     const int sc = row_scale ? (dtype == DMOE_FP16 ? 2 : 1) : 0;
-#define DMOE_PERMUTE_LAUNCH(MAPT, SC)                                                                              \
-    hipLaunchKernelGGL((permute_kernel<MAPT, SC>), dim3((unsigned)nblk), dim3(kBlock), 0, s, (const u32x4 *)in,     \
+    // measured: non-temporal stores are 34 % faster on 403 MB of routed rows (6.7 TB/s moved), within 3 % on 67 MB and
+    // 25 % slower on 201 MB, which the 256 MB Infinity Cache can still hand to the kernel that reads the rows next
+    const bool streamed = R * (int64_t)vecs * 16 > (256ll << 20);
+#define DMOE_PERMUTE_LAUNCH_ONE(MAPT, SC, ST)                                                                      \
+    hipLaunchKernelGGL((permute_kernel<MAPT, SC, ST>), dim3((unsigned)nblk), dim3(kBlock), 0, s, (const u32x4 *)in, \
                        (u32x4 *)out, (const MAPT *)mappings, T, k, R, vecs, nseg, (const uint16_t *)row_scale)
+#define DMOE_PERMUTE_LAUNCH(MAPT, SC)                                                                              \
+    do {                                                                                                            \
+        if (streamed) DMOE_PERMUTE_LAUNCH_ONE(MAPT, SC, true);                                                      \
+        else DMOE_PERMUTE_LAUNCH_ONE(MAPT, SC, false);                                                              \
+    } while (0)
     if (map_type == DMOE_I64) {
         if (sc == 0) DMOE_PERMUTE_LAUNCH(int64_t, 0);
         else if (sc == 1) DMOE_PERMUTE_LAUNCH(int64_t, 1);
@@ -320,6 +333,7 @@ extern "C" int dmoe_permute(const void *in, void *out, const void *mappings, int
         else if (sc == 1) DMOE_PERMUTE_LAUNCH(int32_t, 1);
         else DMOE_PERMUTE_LAUNCH(int32_t, 2);
     }
+#undef DMOE_PERMUTE_LAUNCH_ONE
 #undef DMOE_PERMUTE_LAUNCH
     DMOE_LAUNCH_CHECK("permute_kernel");
     return DMOE_OK;
@@ -423,13 +437,15 @@ extern "C" int dmoe_quant_rows(const void *x, void *q, float *scales, int64_t ro
     DMOE_REQUIRE(rows >= 0 && rows < (1ll << 31), DMOE_ERR_ARG, "dmoe_quant_rows: bad row count");
     if (rows == 0) return DMOE_OK;
     DMOE_REQUIRE(x && q && scales, DMOE_ERR_ARG, "dmoe_quant_rows: null pointer");
-    // the fused permute + quantise kernel without a mapping
-    if (dtype == DMOE_FP16)
-        hipLaunchKernelGGL((permute_quant_kernel<int64_t, true>), dim3((unsigned)rows), dim3(kBlock), 0, (hipStream_t)stream,
-                           (const u32x4 *)x, (uint2 *)q, scales, (const int64_t *)nullptr, 1, rows, vecs);
-    else
-        hipLaunchKernelGGL((permute_quant_kernel<int64_t, false>), dim3((unsigned)rows), dim3(kBlock), 0, (hipStream_t)stream,
-                           (const u32x4 *)x, (uint2 *)q, scales, (const int64_t *)nullptr, 1, rows, vecs);
+    // the fused permute + quantise kernel without a mapping; quantised rows beyond the size of the last-level cache
+    // leave with non-temporal stores (537 MB: 5 % faster)
+    const bool streamed = rows * (int64_t)vecs * 8 > (256ll << 20);
+#define DMOE_QUANT_LAUNCH(HALF, ST)                                                                                    \
+    hipLaunchKernelGGL((permute_quant_kernel<int64_t, HALF, ST>), dim3((unsigned)rows), dim3(kBlock), 0,               \
+                       (hipStream_t)stream, (const u32x4 *)x, (uint2 *)q, scales, (const int64_t *)nullptr, 1, rows, vecs)
+    if (dtype == DMOE_FP16) { if (streamed) DMOE_QUANT_LAUNCH(true, true); else DMOE_QUANT_LAUNCH(true, false); }
+    else { if (streamed) DMOE_QUANT_LAUNCH(false, true); else DMOE_QUANT_LAUNCH(false, false); }
+#undef DMOE_QUANT_LAUNCH
     DMOE_LAUNCH_CHECK("permute_quant_kernel");
     return DMOE_OK;
 }
@@ -449,8 +465,8 @@ extern "C" int dmoe_permute_quant(const void *in, void *q, float *scales, const 
     const int k = (int)(R / T);
     hipStream_t s = (hipStream_t)stream;
 #define DMOE_PQ_LAUNCH(MAPT, HALF)                                                                                     \
-    hipLaunchKernelGGL((permute_quant_kernel<MAPT, HALF>), dim3((unsigned)T), dim3(kBlock), 0, s, (const u32x4 *)in,   \
-                       (uint2 *)q, scales, (const MAPT *)mappings, k, R, vecs)
+    hipLaunchKernelGGL((permute_quant_kernel<MAPT, HALF, false>), dim3((unsigned)T), dim3(kBlock), 0, s,              \
+                       (const u32x4 *)in, (uint2 *)q, scales, (const MAPT *)mappings, k, R, vecs)
     const bool half = dtype == DMOE_FP16;
     if (map_type == DMOE_I64) { if (half) DMOE_PQ_LAUNCH(int64_t, true); else DMOE_PQ_LAUNCH(int64_t, false); }
     else { if (half) DMOE_PQ_LAUNCH(int32_t, true); else DMOE_PQ_LAUNCH(int32_t, false); }

@@ -216,14 +216,19 @@ __global__ __launch_bounds__(kBlock) void permute_quant_kernel(const u32x4 *__re
             amax = fmaxf(amax, fabsf(elem_to_f32<kHalf>((uint16_t)(b[i] >> 16))));
         }
     };
+    // register slots a row of this length fills (the same for every thread): the conversions, 17 instructions per
+    // element, are what bounds this kernel, and a row of 6144 elements fills 3 of the 8 slots
+    const int slots = (vecs + kBlock - 1) / kBlock;
     if (keep) {
 #pragma unroll
         for (int u = 0; u < kKeep; ++u) {
             const int v = threadIdx.x + u * kBlock;
             held[u] = u32x4{0, 0, 0, 0};
             if (v < vecs) held[u] = __builtin_nontemporal_load(src + v);
-            absmax_of(held[u]);
         }
+#pragma unroll
+        for (int u = 0; u < kKeep; ++u)
+            if (u < slots) absmax_of(held[u]);
     } else {
         for (int v = threadIdx.x; v < vecs; v += kBlock) absmax_of(src[v]);
     }
@@ -250,7 +255,8 @@ __global__ __launch_bounds__(kBlock) void permute_quant_kernel(const u32x4 *__re
     if (keep) {
         uint2 out[kKeep];
 #pragma unroll
-        for (int u = 0; u < kKeep; ++u) out[u] = quantised(held[u]);
+        for (int u = 0; u < kKeep; ++u)
+            if (u < slots) out[u] = quantised(held[u]);
         for (int j = 0; j < k; ++j) {
             const int64_t p = map ? load_map(map, tok * k + j) : tok;   // no mapping: rows stay where they are
             if (p < 0 || p >= R) continue;

@@ -189,7 +189,8 @@ __global__ __launch_bounds__(kBlock) void combine_kernel(const u32x4 *__restrict
             u32x4 r;
 #pragma unroll
             for (int i = 0; i < 4; ++i)
-                r[i] = (uint32_t)f32_to_elem<kHalf>(acc[u][2 * i]) | ((uint32_t)f32_to_elem<kHalf>(acc[u][2 * i + 1]) << 16);
+                r[i] = kHalf ? (uint32_t)f32_to_half_bits(acc[u][2 * i]) | ((uint32_t)f32_to_half_bits(acc[u][2 * i + 1]) << 16)
+                             : pack_bf16x2(acc[u][2 * i], acc[u][2 * i + 1]);   // one instruction for the pair
             dst[v] = r;
         }
     }

@@ -67,8 +67,9 @@ def _cpu_baseline(w, x, ids, gates, layer, budget_s: float = 12.0):
     about ``budget_s`` seconds are spent; returns the record of the largest sample."""
     import torch
     from oracle import cpu_path
-    cores = min(os.cpu_count() or 1, 16)
-    torch.set_num_threads(cores)
+    # the threads the environment grants this process: OMP_NUM_THREADS where it is set (a GPU box shares its host
+    # cores between its GPUs), every core otherwise
+    cores = torch.get_num_threads()
     w13 = layer.w13_weight.detach().cpu()
     w2 = layer.w2_weight.detach().cpu()
     xc, idc, gc = x.cpu(), ids.cpu(), gates.cpu()

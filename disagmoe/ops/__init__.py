@@ -1,0 +1,1 @@
+"""Expert-worker part of the reference package of the same name."""

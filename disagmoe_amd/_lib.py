@@ -6,11 +6,11 @@ import os
 from ctypes import c_char_p, c_int, c_int64, c_size_t, c_void_p, POINTER
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-# DMOE_HIP_LIB selects an experimental build of the same library (tuning only)
-LIB_PATH = os.environ.get("DMOE_HIP_LIB") or os.path.join(_HERE, "libdmoe_hip.so")
+LIB_PATH = os.path.join(_HERE, "libdmoe_hip.so")
 
 # dmoe.h constants
 OK = 0
+ERR_ARG, ERR_SHAPE, ERR_DTYPE, ERR_WORKSPACE, ERR_HIP = -1, -2, -3, -4, -5
 BF16, FP16, FP8_E4M3, FP32 = 0, 1, 2, 3
 I32, I64 = 4, 8
 ORDER_REFERENCE, ORDER_STABLE = 0, 1

@@ -33,8 +33,8 @@ def _hipcc() -> str:
 
 
 def build(verbose: bool = True, jobs: int = 4, extra_flags=(), out: str = LIB_PATH, tag: str = "") -> str:
-    """Compile and link; ``extra_flags``/``out``/``tag`` build an experimental copy
-    next to the default library (select it with the DMOE_HIP_LIB environment variable)."""
+    """Compile and link.  ``extra_flags``/``out``/``tag`` build a second copy of the library next to the default
+    one (its objects go to ``build<tag>/``)."""
     hipcc = _hipcc()
     objdir = os.path.join(HERE, "build" + tag)
     os.makedirs(objdir, exist_ok=True)
@@ -68,10 +68,4 @@ def build(verbose: bool = True, jobs: int = 4, extra_flags=(), out: str = LIB_PA
 
 
 if __name__ == "__main__":
-    import argparse
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--tag", default="", help="suffix of an experimental library (libdmoe_hip<tag>.so)")
-    ap.add_argument("flags", nargs="*", help="extra hipcc flags, e.g. -DDMOE_SWZ_MODE=1")
-    a, unknown = ap.parse_known_args()
-    target = LIB_PATH if not a.tag else LIB_PATH.replace(".so", a.tag + ".so")
-    print(build(extra_flags=tuple(a.flags) + tuple(unknown), out=target, tag=a.tag))
+    print(build())

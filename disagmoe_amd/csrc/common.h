@@ -37,9 +37,10 @@ int fail(int code, const char *fmt, ...);
 
 int device_cus();  // compute units of the current device, cached per device
 
-// True the first time it is called with `seen` on the current device (a function attribute such as the dynamic
-// LDS size is set per device).
-bool first_on_device(unsigned long long *seen);
+// Raises a kernel's dynamic LDS limit to `bytes` on the current device, once per device: `seen` is the caller's
+// record of the devices done (a static, one per kernel).  Serialised, and a device is recorded only after the call
+// succeeded, so no thread launches before the attribute is in place and a failure is retried by the next launch.
+hipError_t raise_dynamic_lds(const void *kernel, int bytes, unsigned long long *seen);
 
 __device__ __forceinline__ int lane_id() { return threadIdx.x & (kWave - 1); }
 

@@ -25,12 +25,9 @@ namespace dmoe {
 
 constexpr int kRowBytes = 128;     // bytes of K per tile row in LDS
 
-#ifndef DMOE_SWZ_MODE
-#define DMOE_SWZ_MODE 1
-#endif
-// XOR applied to the 16-byte chunk index of a 128-byte LDS row.  Both forms have
-// a period of at most 32 rows, so fragment rows 32 apart differ by a constant.
-__device__ __forceinline__ int swz(int row) { return DMOE_SWZ_MODE == 0 ? (row & 7) : ((row >> 1) & 7); }
+// XOR applied to the 16-byte chunk index of a 128-byte LDS row.  Its period is
+// 16 rows, so fragment rows 32 apart differ by a constant.
+__device__ __forceinline__ int swz(int row) { return (row >> 1) & 7; }
 __device__ __forceinline__ int lds_off(int row, int chunk) { return row * kRowBytes + ((chunk ^ swz(row)) << 4); }
 
 template <int BM, int BN, int WM, int WN, bool TRANS_B, bool SWIGLU, bool FP8>
@@ -313,10 +310,7 @@ void gmm_kernel(const GmmArgs p) {
             // Two waves share a SIMD.  The two halves of the workgroup run half a step apart: while one
             // half issues its LDS/global traffic for a step, the other half issues the MFMAs of its step,
             // and the barriers hand the roles over.  Waves w and w + 4 sit on the same SIMD.
-#ifndef DMOE_PP_GROUP_MODE
-#define DMOE_PP_GROUP_MODE 0
-#endif
-            const int grp = DMOE_PP_GROUP_MODE == 0 ? (wave >> 2) : (wave & 1);
+            const int grp = wave >> 2;
             if (grp == 1) __syncthreads();
             for (int kt = 0; kt < KT; ++kt) {
                 const int cur = kt & 1;
@@ -400,8 +394,7 @@ static int launch_one(const GmmArgs &args, hipStream_t stream) {
     const size_t lds = 2 * (size_t)(BM + BN) * kRowBytes;
     auto kern = gmm_kernel<BM, BN, WM, WN, TRANS_B, SWIGLU, FP8>;
     static unsigned long long configured = 0;   // devices on which the kernel's LDS size has been raised
-    if (first_on_device(&configured))
-        DMOE_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    DMOE_HIP(raise_dynamic_lds((const void *)kern, (int)lds, &configured));
     const int n_out = SWIGLU ? args.N / 2 : args.N;
     const long long n_tiles = (n_out + BNO - 1) / BNO;
     const long long m_tiles_max = args.rows / BM + args.E;  // sum of ceil(n_e / BM) never exceeds this
@@ -417,9 +410,6 @@ static int launch_one(const GmmArgs &args, hipStream_t stream) {
 }
 
 static int g_variant = 0;  // tuning hook, see dmoe_gmm_tune
-
-static int g_debug_mode = 0;
-int debug_mode() { return g_debug_mode; }
 
 int next_sched_slot() {
     static std::atomic<unsigned int> counter{0};
@@ -473,9 +463,6 @@ static int check_gmm(const char *who, const void *a, const void *b, const void *
 using namespace dmoe;
 
 extern "C" int dmoe_gmm_tune(int variant) {
-#ifdef DMOE_DEBUG_HOOKS
-    if (variant >= 100) { g_debug_mode = variant - 100; return DMOE_OK; }
-#endif
     DMOE_REQUIRE(variant >= 0 && variant <= 8, DMOE_ERR_ARG, "dmoe_gmm_tune: variant %d outside [0, 8]", variant);
     g_variant = variant;
     return DMOE_OK;

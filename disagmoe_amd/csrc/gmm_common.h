@@ -29,9 +29,7 @@ struct GmmArgs {
     int N;          // columns of b per expert (2*I for the swiglu form)
     int ldc;        // columns of c (N, or I for the swiglu form)
     int sched_slot; // entry of the work-counter ring used by this launch
-    int dbg;        // timing experiments, only honoured by builds with DMOE_DEBUG_HOOKS (wrong results)
 };
-int debug_mode();
 
 // ---- work distribution ---------------------------------------------------------------------------
 // Tiles differ in cost (an expert's last m-tile may hold a few rows), so workgroups draw work items from

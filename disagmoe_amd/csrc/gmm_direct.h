@@ -141,11 +141,7 @@ void gmm_direct_kernel(const GmmArgs p) {
     // tile column slot (0..255) -> column of b; slots past the end read the first column (never stored)
     auto b_col = [&](int slot) {
         const int rh = (SWIGLU && slot >= kDN / 2) ? slot - kDN / 2 : slot;
-#ifdef DMOE_DEBUG_HOOKS
-        const int nb = p.dbg == 4 ? 0 : n0;   // timing experiment 4: every n-tile reads the first weight tile
-#else
         const int nb = n0;
-#endif
         const int base = (SWIGLU && slot >= kDN / 2) ? n_out + nb : nb;
         return base + (rh < n_out - n0 ? rh : 0);
     };
@@ -177,10 +173,6 @@ void gmm_direct_kernel(const GmmArgs p) {
     // copy number c (0 .. kLoads-1) of this wavefront for stage s: first its CA blocks of A, then its CB blocks of B
     auto issue_copy = [&](int s, auto c_tag) {
         constexpr int c = decltype(c_tag)::value;
-#ifdef DMOE_DEBUG_HOOKS
-        // timing experiments (wrong results): 1 = no copies after the prologue, 2 = no A copies, 3 = no B copies
-        if (s >= kStages && (p.dbg == 1 || (p.dbg == 2 && c < CA) || (p.dbg == 3 && c >= CA))) return;
-#endif
         const uint32_t lds = smem_addr + (s % kStages) * kStage + cw * 1024;
         if constexpr (c < CA) {
             copy_g2lds_16<c * kBlock>(a_off[c], a_base + (uint64_t)s * 64, lds);
@@ -305,10 +297,6 @@ void gmm_direct_kernel(const GmmArgs p) {
         }
     }
 
-#ifdef DMOE_DEBUG_HOOKS
-    unsigned long long dbg_sum[6] = {0, 0, 0, 0, 0, 0}, dbg_t[5] = {0, 0, 0, 0, 0};
-    const bool dbg_rec = (p.dbg == 21 || p.dbg == 22) && blockIdx.x == 8;
-#endif
     while (q < total) {
         // results of this tile go here after the next tile's copies have been issued
         const int cur_row0 = row0, cur_rows_e = rows_e, cur_n0 = n0, cur_e = e;
@@ -343,14 +331,8 @@ void gmm_direct_kernel(const GmmArgs p) {
 
         // stage 0 of this tile has landed (its other prologue stages, and stores of the previous tile's
         // epilogue that were issued after them, may still be in flight: waiting for fewer is only stricter)
-#ifdef DMOE_DEBUG_HOOKS
-        if (dbg_rec) dbg_t[0] = __builtin_amdgcn_s_memtime();
-#endif
         if constexpr (NP == 0) wait_ahead(pre - 1);
         __syncthreads();
-#ifdef DMOE_DEBUG_HOOKS
-        if (dbg_rec) dbg_t[1] = __builtin_amdgcn_s_memtime();
-#endif
 #pragma unroll
         for (int r = 0; r < NR; ++r) load_frag(0, 0, 0, r);
 
@@ -388,18 +370,11 @@ void gmm_direct_kernel(const GmmArgs p) {
                 });
             }
             if (kSteady || next) {
-#ifdef DMOE_DEBUG_HOOKS
-                if (kSteady && p.dbg == 13) {}   // timing experiment (wrong results): no wait for the copies
-                else
-#endif
                 if constexpr (NP > 0) {}   // the copying wavefronts wait for the data
                 else if constexpr (kSteady) DMOE_WAIT_VMCNT((kStages - 2) * kLoads);
                 else wait_ahead(ahead);
                 __syncthreads();
                 __builtin_amdgcn_sched_barrier(0);
-#ifdef DMOE_DEBUG_HOOKS
-                if (dbg_rec && (s == 0 || s == 3)) dbg_t[s == 0 ? 2 : 3] = __builtin_amdgcn_s_memtime();
-#endif
             }
             static_for<0, NM>([&](auto t_tag) {
                 constexpr int t = decltype(t_tag)::value;
@@ -459,9 +434,6 @@ void gmm_direct_kernel(const GmmArgs p) {
             q = s_item;        // the next work item, written by them before the barrier
         }
 
-#ifdef DMOE_DEBUG_HOOKS
-        if (dbg_rec) dbg_t[4] = __builtin_amdgcn_s_memtime();
-#endif
         auto epilogue = [&]() {
             // ---- epilogue of the finished tile ----
             // The MFMAs take the B fragment as their first operand, so an accumulator holds the tile transposed:
@@ -573,10 +545,6 @@ void gmm_direct_kernel(const GmmArgs p) {
                                     const int grow = wm * TM + i * 32 + row;
                                     const int gcol = col0 + (j - (CW - 1)) * 32 + c * 8;
                                     if (grow >= cur_rows_e || gcol >= n_out) continue;
-#ifdef DMOE_DEBUG_HOOKS
-                                    // timing experiment 8: the epilogue without its stores (a value that never occurs)
-                                    if (p.dbg == 8 && val[0] != 0x7fc17fc1u) continue;
-#endif
                                     *(u32x4 *)((uint16_t *)p.c + (long long)(cur_row0 + grow) * p.ldc + gcol) = val;
                                 }
                             }
@@ -590,25 +558,7 @@ void gmm_direct_kernel(const GmmArgs p) {
             }
     
         };
-#ifdef DMOE_DEBUG_HOOKS
-        if (p.dbg == 6) return;   // timing experiment: results not stored
-#endif
-#ifdef DMOE_DEBUG_HOOKS
-        if (p.dbg == 22) {}   // timing experiment: where the time of a tile goes, without the epilogue
-        else
-#endif
         epilogue();
-#ifdef DMOE_DEBUG_HOOKS
-        if (dbg_rec) {
-            const unsigned long long t5 = __builtin_amdgcn_s_memtime();
-            dbg_sum[0] += dbg_t[1] - dbg_t[0];   // wait for stage 0
-            dbg_sum[1] += dbg_t[2] - dbg_t[1];   // stage 0 up to its hand-over
-            dbg_sum[2] += dbg_t[3] - dbg_t[2];   // stages 1 .. 3
-            dbg_sum[3] += dbg_t[4] - dbg_t[3];   // rest of the main loop
-            dbg_sum[4] += t5 - dbg_t[4];         // epilogue
-            dbg_sum[5] += 1;
-        }
-#endif
         };   // run_tile
         // fp8: one instance per wavefront number (the MFMA slots of its copies are compile-time constants)
         auto run_build = [&](auto guard_tag) {
@@ -643,12 +593,6 @@ void gmm_direct_kernel(const GmmArgs p) {
         if constexpr (NP == 0) next_item();
         else if (q < total) locate_tile(q);
     }
-#ifdef DMOE_DEBUG_HOOKS
-    if (dbg_rec && tid == 0 && dbg_sum[5] > 0)
-        printf("[dbg %d] tiles %llu; per tile (clk): wait for stage 0 %llu, stage 0 %llu, stages 1-3 %llu, rest of the loop %llu, epilogue %llu\n",
-               p.dbg, dbg_sum[5], dbg_sum[0] / dbg_sum[5], dbg_sum[1] / dbg_sum[5], dbg_sum[2] / dbg_sum[5],
-               dbg_sum[3] / dbg_sum[5], dbg_sum[4] / dbg_sum[5]);
-#endif
     sched_finish(p.sched_slot);
 }
 
@@ -659,8 +603,7 @@ static int launch_direct_one(const GmmArgs &args, hipStream_t stream) {
     const size_t lds = (size_t)kStages * (kDM * kDK * 2 + kStageB);
     auto kern = gmm_direct_kernel<kDM, NW, WM, TRANS_B, SWIGLU, FP8, NP>;
     static unsigned long long configured = 0;   // devices on which the kernel's LDS size has been raised
-    if (first_on_device(&configured))
-        DMOE_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    DMOE_HIP(raise_dynamic_lds((const void *)kern, (int)lds, &configured));
     const int n_out = SWIGLU ? args.N / 2 : args.N;
     const long long n_tiles = (n_out + BNO - 1) / BNO;
     const long long m_tiles_max = args.rows / kDM + args.E;
@@ -670,7 +613,6 @@ static int launch_direct_one(const GmmArgs &args, hipStream_t stream) {
     grid = (grid + kXcds - 1) / kXcds * kXcds;   // whole rows of XCDs: the tile order is XCD-aware only then
     GmmArgs launch_args = args;
     launch_args.sched_slot = next_sched_slot();
-    launch_args.dbg = debug_mode();
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3((NW + NP) * 64), lds, stream, launch_args);
     DMOE_LAUNCH_CHECK("gmm_direct_kernel");
     return DMOE_OK;

@@ -17,6 +17,8 @@
 #include <stdarg.h>
 #include <string.h>
 
+#include <mutex>
+
 #include "common.h"
 
 namespace dmoe {
@@ -45,12 +47,17 @@ int device_cus() {
     return cached[dev];
 }
 
-bool first_on_device(unsigned long long *seen) {
+hipError_t raise_dynamic_lds(const void *kernel, int bytes, unsigned long long *seen) {
+    static std::mutex mu;
     int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess) return true;
+    hipError_t err = hipGetDevice(&dev);
+    if (err != hipSuccess) return err;
     const unsigned long long bit = 1ull << (dev & 63);
-    const unsigned long long before = __atomic_fetch_or(seen, bit, __ATOMIC_RELAXED);
-    return (before & bit) == 0;
+    std::lock_guard<std::mutex> lock(mu);
+    if (*seen & bit) return hipSuccess;
+    err = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (err == hipSuccess) *seen |= bit;
+    return err;
 }
 
 constexpr int kChunk = 512;       // rows per wavefront

@@ -23,15 +23,20 @@ def expert_layer_forward(experts: torch.nn.Module, x: torch.Tensor, topk_ids: to
                          order: int = _lib.ORDER_REFERENCE) -> torch.Tensor:
     """``x [T, d]`` bf16, ``topk_ids [T, k]`` int, ``topk_weights [T, k]`` fp32 ->
     ``[T, d]``: ``out[i] = sum_j w[i, j] * FFN_{ids[i, j]}(x[i])``.  ``stages`` (if
-    given) receives the intermediate tensors."""
+    given) receives the intermediate tensors of the kernels that ran; it does not change which
+    kernels run."""
     T, k = topk_ids.shape
     num_experts = experts.num_experts
     mappings, batch_sizes, offsets = memory.route_tokens(topk_ids, num_experts, order)
-    if hasattr(experts, "forward_quantized") and stages is None:
+    if hasattr(experts, "forward_quantized"):
         # fp8 experts: the routed rows are quantised on their way into the expert-sorted buffer
         xq, xs = memory.permute_quantize(x, mappings)
         expert_out = experts.forward_quantized(T * k, xq, xs, batch_sizes)
-        return memory.combine_tokens(expert_out, mappings, topk_weights)
+        out = memory.combine_tokens(expert_out, mappings, topk_weights)
+        if stages is not None:
+            stages.update(mappings=mappings, batch_sizes=batch_sizes, offsets=offsets, permuted_q=xq,
+                          permuted_scale=xs, expert_out=expert_out)
+        return out
     permuted = memory.permute_tokens_cuda(x, mappings)
     expert_out = experts.forward(T * k, permuted, batch_sizes)
     out = memory.combine_tokens(expert_out, mappings, topk_weights)

@@ -77,16 +77,25 @@ def route_tokens(exp_ids: torch.Tensor, num_experts: int, order: int = _lib.ORDE
 
 def get_mappings_from_exp_ids(exp_ids: Union[torch.Tensor, List[int]], num_experts: int) -> Tuple[List[int], List[int]]:
     """Reference signature and return types (memory.py:34-54): Python lists
-    ``(mappings, exp_cnt)``; the counting sort itself runs on the device and the
-    lists are read back (the reference's ``.tolist()`` is the same sync point)."""
-    device = _device_of(exp_ids)
-    if not torch.is_tensor(exp_ids):
-        exp_ids = torch.tensor(exp_ids, dtype=torch.int64)
-    ids = exp_ids.reshape(-1)
-    if ids.numel() and (int(ids.min()) < 0 or int(ids.max()) >= num_experts):
-        raise IndexError("list index out of range")  # what the reference's host loop raises
-    mappings, batch_sizes, _ = route_tokens(ids.to(device), num_experts, _lib.ORDER_REFERENCE)
-    return mappings.tolist(), batch_sizes.tolist()
+    ``(mappings, exp_cnt)``.  Ids that live on the host (a list, as the reference's
+    engine passes at engine.py:675, or a CPU tensor) are sorted on the host by the
+    library's ``dmoe_host_mappings``: no upload, no kernel, no read-back.  Ids on the
+    device are sorted there and the lists read back (the reference's ``.tolist()``
+    is the same sync point)."""
+    if torch.is_tensor(exp_ids) and exp_ids.is_cuda:
+        ids = exp_ids.reshape(-1)
+        if ids.numel() and (int(ids.min()) < 0 or int(ids.max()) >= num_experts):
+            raise IndexError("list index out of range")  # what the reference's host loop raises
+        mappings, batch_sizes, _ = route_tokens(ids, num_experts, _lib.ORDER_REFERENCE)
+        return mappings.tolist(), batch_sizes.tolist()
+    from .metadata import host_mappings
+    ids = exp_ids.reshape(-1).tolist() if torch.is_tensor(exp_ids) else list(exp_ids)
+    try:
+        return host_mappings(ids, num_experts)
+    except _lib.DmoeError as err:
+        if err.code == _lib.ERR_ARG:
+            raise IndexError("list index out of range") from None
+        raise
 
 
 def get_mappings_from_exp_ids_cuda(exp_ids: torch.Tensor, num_experts: int):

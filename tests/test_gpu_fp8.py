@@ -9,8 +9,10 @@
   activations the difference is the rounding of the activations to e4m3 (3
   mantissa bits: relative step 2^-4, about 2.6 % rms per element, which a dot
   product of independent terms passes on undiminished).  No fp8-activation kernel
-  can be closer than that; the tests record the figure and bound it at
-  TOL_FP8_ACT."""
+  can be closer than that; the tests record the figure and bound it by what was
+  measured: one GEMM 0.0273 - 0.0304 (bound TOL_FP8_ACT_GEMM), the two-GEMM FFN,
+  whose intermediate rows are rounded to e4m3 as well, 0.049 - 0.053 (bound
+  TOL_FP8_ACT_FFN)."""
 import pytest
 import torch
 
@@ -22,7 +24,10 @@ from helpers import TOL_FP8, announce, dev, max_rel_err, ragged_sizes
 
 pytestmark = pytest.mark.gpu
 
-TOL_FP8_ACT = 8e-2   # activation-rounding noise against the unquantised-activation oracle (see above)
+# activation-rounding noise against the unquantised-activation oracle: the measured figures plus a margin of a few percent
+# of themselves (see above); the stated 3e-2 is asserted against the oracle with the same quantisation points
+TOL_FP8_ACT_GEMM = 3.2e-2
+TOL_FP8_ACT_FFN = 5.6e-2
 
 
 @pytest.mark.parametrize("rows,d", [(1, 16), (17, 64), (300, 1024), (64, 6144), (5, 16384)])
@@ -68,7 +73,7 @@ def test_gmm_fp8(variant, E, R, K, N):
         ref = ffn.gmm(a, fp8.dequantize_weight(wq, w_s), sizes)
         noise = max_rel_err(out, ref)
         print(f"[fp8] gmm vs unquantised-activation oracle: {noise:.4f}")
-        assert noise <= TOL_FP8_ACT, noise
+        assert noise <= TOL_FP8_ACT_GEMM, noise
     finally:
         gg.set_tile_variant(0)
 
@@ -101,37 +106,61 @@ def _fp8_experts_forward(R):
     ref = ffn.moe_experts_forward(x, dq13, dq2, sizes)
     noise = max_rel_err(out, ref)
     print(f"[fp8] FFN vs unquantised-activation oracle: {noise:.4f}")
-    assert noise <= TOL_FP8_ACT, noise
+    assert noise <= TOL_FP8_ACT_FFN, noise
 
 
 def test_c5_full_size_sampled():
+    # the path bench.py times on C5: route -> fused permute + quantise -> fp8 FFN -> combine
     w = workloads.WORKLOADS["C5"]
     announce(test="fp8_c5", T=w.T, d=w.d, I=w.I, E=w.E)
     from disagmoe_amd.expert_layer import expert_layer_forward
+    from oracle import routing, rows as orows
     ids, gates = workloads.make_routing(w)
-    x = workloads.make_activations(w).to(dev())
+    x_cpu = workloads.make_activations(w)
+    x = x_cpu.to(dev())
     w13, w2 = workloads.make_weights(w, dev())
     layer = MoEExpertsFP8(w13, w2)
     del w13, w2
     stages = {}
     out = expert_layer_forward(layer, x, ids.to(dev()), gates.to(dev()), stages=stages)
     torch.cuda.synchronize()
-    cnt = stages["batch_sizes"].cpu().tolist()
+    assert "permuted_q" in stages and "permuted" not in stages      # the fused kernel ran, not permute + quantise
+    m_ref, cnt_ref = routing.get_mappings_from_exp_ids(ids, w.E)
+    assert stages["mappings"].cpu().tolist() == m_ref and stages["batch_sizes"].cpu().tolist() == cnt_ref
+    # (1) the fused permute + quantise kernel at full size, every row, bit for bit
+    xq, xs = stages["permuted_q"].cpu(), stages["permuted_scale"].cpu()
+    inv = torch.empty(w.R, dtype=torch.int64)
+    inv[torch.tensor(m_ref)] = torch.arange(w.R)
+    step = 4096
+    for r0 in range(0, w.R, step):                                  # in slabs: the fp32 copy of all rows is 800 MB
+        q_ref, s_ref = fp8.quantize_rows(x_cpu[inv[r0:r0 + step] // w.k])
+        assert torch.equal(xq[r0:r0 + step].view(torch.uint8), q_ref.view(torch.uint8)), r0
+        assert torch.equal(xs[r0:r0 + step], s_ref), r0
+    # (2) the FFN on sampled rows of every expert
     off = stages["offsets"].cpu().tolist()
-    xp, y = stages["permuted"], stages["expert_out"]
+    y = stages["expert_out"]
     worst = noise = 0.0
     for e in range(w.E):
-        pick = torch.tensor(sorted({off[e], off[e] + cnt[e] - 1, off[e] + cnt[e] // 2, off[e] + 17}), device=dev())
+        n = cnt_ref[e]
+        if n == 0:
+            continue
+        pick = sorted({off[e] + min(i, n - 1) for i in (0, 17, n // 2, n - 1)})
+        rows_in = x_cpu[inv[torch.tensor(pick)] // w.k]
+        sel = torch.tensor(pick, device=dev())
         q13, s13 = layer.w13_q[e:e + 1].cpu(), layer.w13_scale[e:e + 1].cpu()
         q2, s2 = layer.w2_q[e:e + 1].cpu(), layer.w2_scale[e:e + 1].cpu()
-        same_points = fp8.moe_experts_forward_fp8(xp[pick].cpu(), q13, s13, q2, s2, [pick.numel()])
-        worst = max(worst, max_rel_err(y[pick], same_points))
-        ref = ffn.moe_experts_forward(xp[pick].cpu(), fp8.dequantize_weight(q13, s13), fp8.dequantize_weight(q2, s2),
-                                      [pick.numel()])
-        noise = max(noise, max_rel_err(y[pick], ref))
+        same_points = fp8.moe_experts_forward_fp8(rows_in, q13, s13, q2, s2, [len(pick)])
+        worst = max(worst, max_rel_err(y[sel], same_points))
+        ref = ffn.moe_experts_forward(rows_in, fp8.dequantize_weight(q13, s13), fp8.dequantize_weight(q2, s2), [len(pick)])
+        noise = max(noise, max_rel_err(y[sel], ref))
     print(f"[fp8] C5 FFN: same quantisation points {worst:.4f}, unquantised-activation oracle {noise:.4f}")
     assert worst <= TOL_FP8, worst
-    assert noise <= TOL_FP8_ACT, noise
+    assert noise <= TOL_FP8_ACT_FFN, noise
+    # (3) the combine on the expert outputs the device produced
+    sample = torch.arange(0, w.T, 997)
+    m = torch.tensor(m_ref).view(w.T, w.k)[sample]
+    ref_out = (y[m.to(dev())].float() * gates[sample].to(dev())[:, :, None]).sum(1)
+    assert max_rel_err(out[sample.to(dev())], ref_out) <= 1e-2
     assert torch.isfinite(out.float()).all()
 
 
@@ -178,10 +207,11 @@ def test_permute_quantize_bit_exact(T, d, k, E, dtype):
 
 
 def test_fp8_layer_fused_rows_equal_two_step():
-    # the layer quantises the routed rows on their way into the expert-sorted buffer; asking for the intermediate
-    # tensors takes the two-step path: the results have the same bits
+    # the layer quantises the routed rows on their way into the expert-sorted buffer; permute, then quantise inside
+    # the experts' forward, then combine, gives the same bits
     announce(test="fp8_layer_fused_rows")
     from disagmoe_amd.expert_layer import expert_layer_forward
+    from disagmoe_amd.ops import memory
     E, d, I, T, k = 8, 1024, 1536, 300, 2
     g = torch.Generator().manual_seed(17)
     w13 = (torch.randn(E, d, 2 * I, generator=g) * 0.02).to(torch.bfloat16)
@@ -190,6 +220,11 @@ def test_fp8_layer_fused_rows_equal_two_step():
     ids = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(dev())
     gates = torch.softmax(torch.randn(T, k, generator=g), dim=-1).to(dev())
     layer = MoEExpertsFP8(w13.to(dev()), w2.to(dev()))
-    fused = expert_layer_forward(layer, x, ids, gates)
-    two_step = expert_layer_forward(layer, x, ids, gates, stages={})
-    assert torch.equal(fused, two_step)
+    stages = {}
+    fused = expert_layer_forward(layer, x, ids, gates, stages=stages)
+    assert torch.equal(fused, expert_layer_forward(layer, x, ids, gates))      # `stages` does not change the kernels
+    mappings, batch_sizes, _ = memory.route_tokens(ids, E)
+    assert torch.equal(mappings, stages["mappings"])
+    y = layer.forward(T * k, memory.permute_tokens_cuda(x, mappings), batch_sizes)
+    assert torch.equal(y, stages["expert_out"])
+    assert torch.equal(memory.combine_tokens(y, mappings, gates), fused)

@@ -59,7 +59,11 @@ def test_no_cpu_fallback():
     x = torch.zeros(4, 8, dtype=torch.bfloat16)
     with pytest.raises(RuntimeError):
         memory.permute_tokens_cuda(x, [0, 1, 2, 3])
+    # ids that live on the host are sorted by the library's host code, as the reference's host loop does: no device
+    assert memory.get_mappings_from_exp_ids([2, 0, 2, 1, 0, 2], 3) == ([5, 1, 4, 2, 0, 3], [2, 1, 3])
+    with pytest.raises(IndexError):
+        memory.get_mappings_from_exp_ids([0, 3], 3)
     with pytest.raises(RuntimeError):
-        memory.get_mappings_from_exp_ids([0, 1], 2)
+        memory.route_tokens(torch.tensor([0, 1]), 2)
     with pytest.raises(RuntimeError):
         gg.gmm(x, torch.zeros(1, 8, 8, dtype=torch.bfloat16), torch.tensor([4]))

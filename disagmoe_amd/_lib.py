@@ -24,6 +24,9 @@ SIGNATURES = {
     "dmoe_route_scratch_bytes": (c_int, [c_int64, c_int, POINTER(c_size_t)]),
     "dmoe_route": (c_int, [c_void_p, c_int, c_int64, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p,
                            c_void_p, c_size_t, c_void_p]),
+    "dmoe_route_noalloc_max_bytes": (c_int, [POINTER(c_size_t)]),
+    "dmoe_route_noalloc": (c_int, [c_void_p, c_int, c_int64, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p,
+                                   c_void_p]),
     "dmoe_topk_softmax": (c_int, [c_void_p, c_int, c_int64, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p]),
     "dmoe_sort_by_prefill_order": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_void_p]),
     "dmoe_move_row_infos": (c_int, [c_void_p, c_int, c_void_p, c_int64, c_void_p]),

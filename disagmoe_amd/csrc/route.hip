@@ -60,6 +60,11 @@ hipError_t raise_dynamic_lds(const void *kernel, int bytes, unsigned long long *
     return err;
 }
 
+// Scratch of dmoe_route_noalloc: the per-chunk histograms of one routing call.  File scope, one copy per device,
+// held until the process ends.  Host code reaches it only through the address hipGetSymbolAddress returns.
+constexpr size_t kStaticScratchBytes = 4u << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
 constexpr int kChunk = 512;       // rows per wavefront
 constexpr int kMaxExperts = 4096; // 3 int tables of E entries must fit in LDS
 // chunks that one workgroup takes, a wavefront each, when their tables fit in LDS (measured: 6144 rows 13 us against
@@ -354,6 +359,45 @@ extern "C" int dmoe_route_scratch_bytes(int64_t R, int E, size_t *bytes) {
     // a histogram per chunk and, behind them, the column sums of the scanned form
     *bytes = one_workgroup(nchunks, E) ? 0 : (size_t)(nchunks + 1) * (size_t)E * sizeof(int);
     return DMOE_OK;
+}
+
+// Device address of the file-scope scratch array on the current device (looked up once per device).
+static int static_scratch(void **out) {
+    static std::mutex mu;
+    static void *ptr_of_device[64];
+    int dev = 0;
+    DMOE_HIP(hipGetDevice(&dev));
+    DMOE_REQUIRE(dev >= 0 && dev < 64, DMOE_ERR_ARG, "dmoe_route_noalloc: device ordinal %d outside [0, 64)", dev);
+    std::lock_guard<std::mutex> lock(mu);
+    if (ptr_of_device[dev] == nullptr) {
+        void *ptr = nullptr;
+        DMOE_HIP(hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(dmoe::scratch)));
+        DMOE_REQUIRE(ptr != nullptr, DMOE_ERR_HIP, "dmoe_route_noalloc: no device address for the scratch array");
+        ptr_of_device[dev] = ptr;
+    }
+    *out = ptr_of_device[dev];
+    return DMOE_OK;
+}
+
+extern "C" int dmoe_route_noalloc_max_bytes(size_t *bytes) {
+    DMOE_REQUIRE(bytes != nullptr, DMOE_ERR_ARG, "dmoe_route_noalloc_max_bytes: null output");
+    *bytes = kStaticScratchBytes;
+    return DMOE_OK;
+}
+
+extern "C" int dmoe_route_noalloc(const void *ids, int ids_type, int64_t R, int E, int order, void *mappings,
+                                  int map_type, int64_t *batch_sizes, int64_t *offsets, void *stream) {
+    size_t need = 0;
+    int rc = dmoe_route_scratch_bytes(R, E, &need);
+    if (rc != DMOE_OK) return rc;
+    DMOE_REQUIRE(need <= kStaticScratchBytes, DMOE_ERR_WORKSPACE,
+                 "dmoe_route_noalloc: R=%lld rows over E=%d experts need %zu bytes of scratch, the built-in buffer holds %zu "
+                 "(use dmoe_route with a caller-owned buffer)", (long long)R, E, need, (size_t)kStaticScratchBytes);
+    void *ptr = nullptr;
+    rc = static_scratch(&ptr);
+    if (rc != DMOE_OK) return rc;
+    // every entry of the histograms that a launch reads has been written by the launch before it: nothing to clear
+    return dmoe_route(ids, ids_type, R, E, order, mappings, map_type, batch_sizes, offsets, ptr, kStaticScratchBytes, stream);
 }
 
 extern "C" int dmoe_route(const void *ids, int ids_type, int64_t R, int E, int order, void *mappings, int map_type,

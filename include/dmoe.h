@@ -78,6 +78,21 @@ int dmoe_route(const void *ids, int ids_type, int64_t R, int E, int order,
                void *mappings, int map_type, int64_t *batch_sizes, int64_t *offsets,
                void *scratch, size_t scratch_bytes, void *stream);
 
+/* dmoe_route for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in
+ * the reference.  Same arguments and results as dmoe_route without the scratch
+ * buffer: the per-chunk histograms live in a buffer built into the library, one copy
+ * per device, dmoe_route_noalloc_max_bytes() bytes (4 MiB), held until the process
+ * ends.  The call allocates nothing and frees nothing.  A problem whose
+ * dmoe_route_scratch_bytes(R, E) exceeds that size is refused with
+ * DMOE_ERR_WORKSPACE (4 MiB cover e.g. 8.3 M rows over 64 experts, 130 k rows over
+ * 4096).  All calls on one device share the buffer: calls that overlap in time on
+ * one device (two streams) race; calls on one stream do not. */
+int dmoe_route_noalloc_max_bytes(size_t *bytes);
+int dmoe_route_noalloc(const void *ids, int ids_type, int64_t R, int E, int order,
+                       void *mappings, int map_type, int64_t *batch_sizes, int64_t *offsets,
+                       void *stream);
+
 /* ---- routing producer ---------------------------------------------------
  * dmoe_topk_softmax replaces vllm's fused_topk(hidden_states, gating_output,
  * topk, renormalize) as the attention side calls it

@@ -39,19 +39,24 @@ SIGNATURES = {
     "dmoe_combine": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int64, c_int, c_int64, c_int, c_int,
                              c_void_p]),
     "dmoe_gmm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int64, c_int64, c_int, c_int,
-                         c_void_p]),
+                         c_void_p, c_void_p, c_size_t, c_void_p]),
     "dmoe_gmm_swiglu": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int64, c_int64, c_int,
-                                c_int, c_void_p]),
+                                c_int, c_void_p, c_void_p, c_size_t, c_void_p]),
     "dmoe_gmm_workspace_bytes": (c_int, [c_int, POINTER(c_size_t)]),
-    "dmoe_gmm_tune": (c_int, [c_int]),
     "dmoe_quant_rows": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int, c_void_p]),
     "dmoe_permute_quant": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int,
                                    c_void_p]),
     "dmoe_gmm_fp8": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int64,
-                             c_int64, c_void_p]),
+                             c_int64, c_void_p, c_void_p, c_size_t, c_void_p]),
     "dmoe_gmm_fp8_swiglu": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int,
-                                    c_int64, c_int64, c_void_p]),
+                                    c_int64, c_int64, c_void_p, c_void_p, c_size_t, c_void_p]),
 }
+
+#: exported for the library's own tests and benchmarks, not declared in include/dmoe.h (csrc/tuning.h)
+TEST_HOOKS = {
+    "dmoe_gmm_tune": (c_int, [c_int]),
+}
+GMM_STATE_BYTES = 33024
 
 _lib = None
 
@@ -75,7 +80,7 @@ def load() -> ctypes.CDLL:
             f"{LIB_PATH} is missing: build it with `python -m disagmoe_amd.build` "
             "(hipcc, gfx950). disagmoe_amd has no CPU fallback.")
     lib = ctypes.CDLL(LIB_PATH)
-    for name, (restype, argtypes) in SIGNATURES.items():
+    for name, (restype, argtypes) in {**SIGNATURES, **TEST_HOOKS}.items():
         fn = getattr(lib, name)  # AttributeError if the library does not export it
         fn.restype = restype
         fn.argtypes = argtypes

@@ -17,9 +17,10 @@
 //     its way into LDS so that both MFMA operands are read K-contiguous;
 //   * each wavefront owns a TM x TN sub-tile as FM x FN accumulators of
 //     v_mfma_f32_32x32x16_bf16 (v_mfma_f32_32x32x64_f8f6f4 for fp8).
-#include <atomic>
+#include <mutex>
 
 #include "gmm_common.h"
+#include "tuning.h"
 
 namespace dmoe {
 
@@ -96,14 +97,14 @@ void gmm_kernel(const GmmArgs p) {
     __shared__ long long s_item;
     const int streams = (G % kXcds == 0) ? kXcds : 1;
     unsigned int draw = 0;
-    if (tid == 0) draw = sched_draw(p.sched_slot, streams);
+    if (tid == 0) draw = sched_draw(p.sched, streams);
     for (;;) {
         if (tid == 0) s_item = sched_item(draw, streams);
         __syncthreads();
         const long long q = s_item;
         if (q >= total) break;
-        if (tid == 0) draw = sched_draw(p.sched_slot, streams);   // next item; the round trip hides behind this tile
-        const TileCoord tc = decode_tile<BM>(q, G, total, n_tiles, E, s_tile_start, s_row_start);
+        if (tid == 0) draw = sched_draw(p.sched, streams);   // next item; the round trip hides behind this tile
+        const TileCoord tc = decode_tile<BM>(item_order(q, G, total), n_tiles, E, s_tile_start, s_row_start);
         const int e = tc.e, nt = tc.nt, row0 = tc.row0, rows_e = tc.rows_e;
         const int n0 = nt * BNO;                               // first output column
 
@@ -384,7 +385,7 @@ void gmm_kernel(const GmmArgs p) {
             }
         }
     }
-    sched_finish(p.sched_slot);
+    sched_finish(p.sched);
 }
 
 template <int BM, int BN, int WM, int WN, bool TRANS_B, bool SWIGLU, bool FP8>
@@ -402,18 +403,65 @@ static int launch_one(const GmmArgs &args, hipStream_t stream) {
     if (m_tiles_max * n_tiles < grid) grid = m_tiles_max * n_tiles;
     if (grid < 1) grid = 1;
     grid = (grid + kXcds - 1) / kXcds * kXcds;   // whole rows of XCDs: the tile order is XCD-aware only then
-    GmmArgs launch_args = args;
-    launch_args.sched_slot = next_sched_slot();
-    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NT), lds, stream, launch_args);
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NT), lds, stream, args);
     DMOE_LAUNCH_CHECK("gmm_kernel");
     return DMOE_OK;
 }
 
 static int g_variant = 0;  // tuning hook, see dmoe_gmm_tune
 
-int next_sched_slot() {
-    static std::atomic<unsigned int> counter{0};
-    return (int)(counter.fetch_add(1, std::memory_order_relaxed) % kSchedSlots);
+// ---- where a launch keeps its counters ----------------------------------------------------------------
+// With a state block of the caller: there, the split tiles' arrival counters behind them, and the partial sums in
+// the caller's workspace.  Without one: in a slot of the library's own, one per stream per device (launches on one stream do not overlap, launches on
+// different streams get different slots); nothing is split then.  A launch that is being recorded into a graph may
+// be replayed on any stream at any time, so it must bring its own state block.
+constexpr int kOwnSlots = 64;
+static __device__ SchedSlot g_own_slots[kOwnSlots];
+
+static int own_slot(hipStream_t stream, SchedSlot **out) {
+    struct Entry { int dev; hipStream_t stream; };
+    static std::mutex mu;
+    static Entry table[64][kOwnSlots];
+    static int used[64];
+    static SchedSlot *base[64];
+    int dev = 0;
+    DMOE_HIP(hipGetDevice(&dev));
+    DMOE_REQUIRE(dev >= 0 && dev < 64, DMOE_ERR_ARG, "grouped GEMM: device ordinal %d outside [0, 64)", dev);
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &capture) != hipSuccess) (void)hipGetLastError();
+    DMOE_REQUIRE(capture == hipStreamCaptureStatusNone, DMOE_ERR_WORKSPACE,
+                 "grouped GEMM: a launch recorded into a graph needs a caller-owned state block (DMOE_GMM_STATE_BYTES)");
+    std::lock_guard<std::mutex> lock(mu);
+    if (base[dev] == nullptr) {
+        void *ptr = nullptr;
+        DMOE_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_own_slots)));
+        base[dev] = (SchedSlot *)ptr;
+    }
+    int slot = -1;
+    for (int i = 0; i < used[dev]; ++i)
+        if (table[dev][i].stream == stream) { slot = i; break; }
+    if (slot < 0) {
+        DMOE_REQUIRE(used[dev] < kOwnSlots, DMOE_ERR_WORKSPACE,
+                     "grouped GEMM: more than %d streams on device %d without a state block; pass one", kOwnSlots, dev);
+        slot = used[dev]++;
+        table[dev][slot] = Entry{dev, stream};
+    }
+    *out = base[dev] + slot;
+    return DMOE_OK;
+}
+
+static int bind_state(GmmArgs &args, void *state, void *workspace, size_t workspace_bytes, hipStream_t stream) {
+    args.arrive = nullptr; args.partials = nullptr; args.partial_bytes = 0;
+    if (state == nullptr) return own_slot(stream, &args.sched);
+    DMOE_REQUIRE(((uintptr_t)state & 255) == 0, DMOE_ERR_WORKSPACE, "grouped GEMM: the state block must be 256-byte aligned");
+    args.sched = (SchedSlot *)state;
+    if (workspace != nullptr && workspace_bytes > 0) {
+        DMOE_REQUIRE(((uintptr_t)workspace & 15) == 0, DMOE_ERR_WORKSPACE, "grouped GEMM: the workspace must be 16-byte aligned");
+        args.arrive = (unsigned int *)((char *)state + kWsArriveOffset);
+        args.partials = (float *)workspace;
+        args.partial_bytes = (long long)workspace_bytes;
+    }
+    return DMOE_OK;
 }
 
 template <bool TRANS_B, bool SWIGLU, bool FP8>
@@ -431,7 +479,7 @@ static int launch_by_rows(const GmmArgs &args, hipStream_t stream) {
     // a tile size that would leave more than half of the CUs without a tile is halved (small problems: latency counts)
     const long long n_tiles = ((SWIGLU ? args.N / 2 : args.N) + (SWIGLU ? 127 : 255)) / (SWIGLU ? 128 : 256);
     while (tile_rows > 64 && (args.rows / tile_rows + (args.E + 1) / 2) * n_tiles * 2 < device_cus()) tile_rows /= 2;
-    if (g_variant >= 5) tile_rows = g_variant == 5 ? 64 : (g_variant == 6 ? 128 : (g_variant == 7 ? 256 : 260));   // direct kernel, fixed tile rows (260: 256 rows on 4 wavefronts)
+    if (g_variant >= 5) tile_rows = g_variant == 5 ? 64 : (g_variant == 6 ? 128 : 256);   // direct kernel, fixed tile rows
     if constexpr (!FP8) {
         // global -> LDS direct path: whole stages of 32 k, 32-bit offsets inside one expert's weights
         if (args.K % 32 == 0 && (long long)args.K * args.N * 2 < (1ll << 32))
@@ -463,7 +511,7 @@ static int check_gmm(const char *who, const void *a, const void *b, const void *
 using namespace dmoe;
 
 extern "C" int dmoe_gmm_tune(int variant) {
-    DMOE_REQUIRE(variant >= 0 && variant <= 8, DMOE_ERR_ARG, "dmoe_gmm_tune: variant %d outside [0, 8]", variant);
+    DMOE_REQUIRE(variant >= 0 && variant <= 7, DMOE_ERR_ARG, "dmoe_gmm_tune: variant %d outside [0, 7]", variant);
     g_variant = variant;
     return DMOE_OK;
 }
@@ -471,49 +519,61 @@ extern "C" int dmoe_gmm_tune(int variant) {
 extern "C" int dmoe_gmm_workspace_bytes(int E, size_t *bytes) {
     DMOE_REQUIRE(bytes != nullptr, DMOE_ERR_ARG, "dmoe_gmm_workspace_bytes: null output");
     DMOE_REQUIRE(E > 0 && E <= kMaxGroups, DMOE_ERR_SHAPE, "dmoe_gmm_workspace_bytes: E=%d outside [1, %d]", E, kMaxGroups);
-    *bytes = 256;  // the work list lives in LDS; a token allocation keeps the reference's calling pattern valid
+    // room for the partial sums of two pieces per compute unit (a piece of a 256 x 256 tile is 256 KiB of fp32)
+    *bytes = (size_t)2 * (size_t)device_cus() * 256 * 256 * sizeof(float);
     return DMOE_OK;
 }
 
 extern "C" int dmoe_gmm(const void *a, const void *b, void *c, const int64_t *batch_sizes, int64_t rows, int E,
-                        int64_t K, int64_t N, int trans_b, int dtype, void *stream) {
+                        int64_t K, int64_t N, int trans_b, int dtype, void *state, void *workspace,
+                        size_t workspace_bytes, void *stream) {
     DMOE_REQUIRE(dtype == DMOE_BF16, DMOE_ERR_DTYPE, "dmoe_gmm: dtype %d (bf16 only)", dtype);
     int rc = check_gmm("dmoe_gmm", a, b, c, batch_sizes, rows, E, K, N, 8);
     if (rc != DMOE_OK) return rc;
     if (rows == 0) return DMOE_OK;
     GmmArgs args{(const char *)a, (const char *)b, (char *)c, batch_sizes, nullptr, nullptr, rows, E, (int)K, (int)N, (int)N};
+    rc = bind_state(args, state, workspace, workspace_bytes, (hipStream_t)stream);
+    if (rc != DMOE_OK) return rc;
     return trans_b ? launch_by_rows<true, false, false>(args, (hipStream_t)stream)
                    : launch_by_rows<false, false, false>(args, (hipStream_t)stream);
 }
 
 extern "C" int dmoe_gmm_swiglu(const void *a, const void *b, void *h, const int64_t *batch_sizes, int64_t rows, int E,
-                               int64_t K, int64_t I, int trans_b, int dtype, void *stream) {
+                               int64_t K, int64_t I, int trans_b, int dtype, void *state, void *workspace,
+                               size_t workspace_bytes, void *stream) {
     DMOE_REQUIRE(dtype == DMOE_BF16, DMOE_ERR_DTYPE, "dmoe_gmm_swiglu: dtype %d (bf16 only)", dtype);
     int rc = check_gmm("dmoe_gmm_swiglu", a, b, h, batch_sizes, rows, E, K, I, 8);
     if (rc != DMOE_OK) return rc;
     if (rows == 0) return DMOE_OK;
     GmmArgs args{(const char *)a, (const char *)b, (char *)h, batch_sizes, nullptr, nullptr, rows, E, (int)K, (int)(2 * I), (int)I};
+    rc = bind_state(args, state, workspace, workspace_bytes, (hipStream_t)stream);
+    if (rc != DMOE_OK) return rc;
     return trans_b ? launch_by_rows<true, true, false>(args, (hipStream_t)stream)
                    : launch_by_rows<false, true, false>(args, (hipStream_t)stream);
 }
 
 extern "C" int dmoe_gmm_fp8(const void *a, const float *a_scale, const void *b, const float *b_scale, void *c,
-                            const int64_t *batch_sizes, int64_t rows, int E, int64_t K, int64_t N, void *stream) {
+                            const int64_t *batch_sizes, int64_t rows, int E, int64_t K, int64_t N, void *state,
+                            void *workspace, size_t workspace_bytes, void *stream) {
     int rc = check_gmm("dmoe_gmm_fp8", a, b, c, batch_sizes, rows, E, K, N, 16);
     if (rc != DMOE_OK) return rc;
     DMOE_REQUIRE(b_scale != nullptr && (rows == 0 || a_scale != nullptr), DMOE_ERR_ARG, "dmoe_gmm_fp8: null scales");
     if (rows == 0) return DMOE_OK;
     GmmArgs args{(const char *)a, (const char *)b, (char *)c, batch_sizes, a_scale, b_scale, rows, E, (int)K, (int)N, (int)N};
+    rc = bind_state(args, state, workspace, workspace_bytes, (hipStream_t)stream);
+    if (rc != DMOE_OK) return rc;
     return launch_by_rows<true, false, true>(args, (hipStream_t)stream);
 }
 
 extern "C" int dmoe_gmm_fp8_swiglu(const void *a, const float *a_scale, const void *b, const float *b_scale, void *h,
                                    const int64_t *batch_sizes, int64_t rows, int E, int64_t K, int64_t I,
-                                   void *stream) {
+                                   void *state, void *workspace, size_t workspace_bytes, void *stream) {
     int rc = check_gmm("dmoe_gmm_fp8_swiglu", a, b, h, batch_sizes, rows, E, K, I, 16);
     if (rc != DMOE_OK) return rc;
     DMOE_REQUIRE(b_scale != nullptr && (rows == 0 || a_scale != nullptr), DMOE_ERR_ARG, "dmoe_gmm_fp8_swiglu: null scales");
     if (rows == 0) return DMOE_OK;
     GmmArgs args{(const char *)a, (const char *)b, (char *)h, batch_sizes, a_scale, b_scale, rows, E, (int)K, (int)(2 * I), (int)I};
+    rc = bind_state(args, state, workspace, workspace_bytes, (hipStream_t)stream);
+    if (rc != DMOE_OK) return rc;
     return launch_by_rows<true, true, true>(args, (hipStream_t)stream);
 }

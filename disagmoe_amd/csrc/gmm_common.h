@@ -28,47 +28,95 @@ struct GmmArgs {
     int K;          // contraction length (elements)
     int N;          // columns of b per expert (2*I for the swiglu form)
     int ldc;        // columns of c (N, or I for the swiglu form)
-    int sched_slot; // entry of the work-counter ring used by this launch
+    // state of the launch in device memory (the caller's state block and workspace, or the library's own counters)
+    struct SchedSlot *sched;      // work counters, zero between launches
+    unsigned int *arrive;         // arrival counters of the split tiles, zero between launches (nullptr: no splitting)
+    float *partials;              // fp32 partial results of the pieces of split tiles
+    long long partial_bytes;      // capacity of `partials`
 };
 
 // ---- work distribution ---------------------------------------------------------------------------
 // Tiles differ in cost (an expert's last m-tile may hold a few rows), so workgroups draw work items from
 // counters instead of striding over them.  There is one counter per XCD (workgroup id % 8): XCD x draws
 // j = 0, 1, 2, ... and works on item q = 8 j + x, which keeps the items that share operand tiles on one
-// L2 (see decode_tile) exactly as a static stride would, while a slow tile no longer holds up the tiles
-// queued behind it.  The counters of a launch live in one entry of a small ring in device memory; the
-// last workgroup to finish clears the entry, so no host-side reset or scratch argument is needed.
-// Launches that run concurrently must not share an entry: the host hands entries out round-robin.
-constexpr int kSchedSlots = 64;
+// L2 (see item_order) exactly as a static stride would, while a slow tile no longer holds up the tiles
+// queued behind it.  The counters of a launch live in device memory that is zero when the launch starts
+// (the caller's state block, or the library's own slot of the launch's stream); the last workgroup
+// to finish clears them again.  Launches that may overlap in time must not share them.
 struct SchedSlot {
     unsigned int next[kXcds];
     unsigned int done;
     unsigned int pad[7];
 };
-static __device__ SchedSlot g_sched[kSchedSlots];
+
+// Layout of a caller-owned state block (DMOE_GMM_STATE_BYTES): work counters, then arrival counters of the split tiles.
+constexpr size_t kWsArriveOffset = 256;
+constexpr int kWsArriveCount = 8 * 1024;                                  // (split tiles) x (wavefronts of a tile)
+static_assert(kWsArriveOffset + kWsArriveCount * sizeof(unsigned int) == DMOE_GMM_STATE_BYTES, "state block as dmoe.h states it");
 
 // Next work item of this workgroup (all threads get the same value), or -1 when its stream is exhausted.
 // `carry` holds the draw made ahead of time by thread 0 (see sched_draw).
-__device__ __forceinline__ unsigned int sched_draw(int slot, int streams) {
-    return atomicAdd(&g_sched[slot].next[streams == 1 ? 0 : (blockIdx.x % kXcds)], 1u);
+__device__ __forceinline__ unsigned int sched_draw(SchedSlot *slot, int streams) {
+    return atomicAdd(&slot->next[streams == 1 ? 0 : (blockIdx.x % kXcds)], 1u);
 }
 __device__ __forceinline__ long long sched_item(unsigned int j, int streams) {
     return streams == 1 ? (long long)j : (long long)j * kXcds + (blockIdx.x % kXcds);
 }
-// Called once per workgroup after its last draw; the last caller of the launch clears the entry.
-__device__ __forceinline__ void sched_finish(int slot) {
+// Called once per workgroup after its last draw; the last caller of the launch clears the counters.
+__device__ __forceinline__ void sched_finish(SchedSlot *slot) {
     if (threadIdx.x == 0) {
         __threadfence();
-        const unsigned int before = atomicAdd(&g_sched[slot].done, 1u);
+        const unsigned int before = atomicAdd(&slot->done, 1u);
         if (before == gridDim.x - 1) {
             // cleared with the same kind of operation the counters are advanced with, so that the clear is
             // seen wherever the next launch's draws are performed
 #pragma unroll
-            for (int i = 0; i < kXcds; ++i) atomicExch(&g_sched[slot].next[i], 0u);
-            atomicExch(&g_sched[slot].done, 0u);
+            for (int i = 0; i < kXcds; ++i) atomicExch(&slot->next[i], 0u);
+            atomicExch(&slot->done, 0u);
             __threadfence();
         }
     }
+}
+
+// ---- the last, partly filled round of tiles ----------------------------------------------------------
+// `tiles` tiles on G workgroups leave the last round with rem = tiles % G tiles: G - rem compute units idle for the
+// length of a tile.  Those rem tiles are therefore cut along K into `split` pieces of equal length, drawn like any
+// other work item after the whole tiles; rem * split pieces fill ceil(rem * split / G) rounds of 1 / split of a
+// tile's length.  A piece leaves its fp32 accumulators in the workspace; the piece of a tile that arrives last adds
+// all of them up in the order of the pieces (so the sum does not depend on which one that is) and writes the result.
+struct WorkPlan {
+    long long tiles;     // (expert, m-tile, n-tile) triples
+    long long whole;     // tiles computed in one piece: items [0, whole)
+    int rem;             // tiles cut in pieces: items [whole, whole + rem * split), piece-major
+    int split;           // pieces per such tile (1: nothing is cut, rem == 0)
+    long long items;     // whole + rem * split
+};
+constexpr int kMaxSplit = 8;
+constexpr int kMaxWholeRounds = 3;
+constexpr int kMinPieceStages = 64;   // shorter pieces lose to their own overhead (measured on 44- and 128-stage tiles)
+
+__device__ __host__ __forceinline__ WorkPlan plan_work(long long tiles, int G, int stages, long long max_pieces, int max_rem) {
+    WorkPlan w;
+    w.tiles = tiles; w.whole = tiles; w.rem = 0; w.split = 1; w.items = tiles;
+    const long long rem = tiles % G;
+    // Launches of many rounds gain nothing (measured: 15.3 rounds of 128 stages): their workgroups are up to a tile
+    // apart by the time the last round starts, and the counters balance that as well as pieces would.
+    if (rem == 0 || rem > max_rem || tiles / G > kMaxWholeRounds) return w;
+    // Time of the remainder in stages.  A work item costs its stages and about 8 more (draw, first copies in flight,
+    // drain, epilogue); a piece also writes its sums past the L2 and counts itself in (about 12), and the last piece of
+    // a tile reads all of them back (4 + 4 per piece).  The smallest wins, if it saves 8 % of a whole tile.
+    int best = 1;
+    const long long whole_cost = stages + 8;
+    long long best_cost = whole_cost;
+    for (int p = 2; p <= kMaxSplit; ++p) {
+        if (rem * p > max_pieces || stages / p < kMinPieceStages) break;
+        const long long rounds = (rem * p + G - 1) / G;
+        const long long cost = rounds * ((stages + p - 1) / p + 20) + 4 + 4 * p;
+        if (cost < best_cost) { best = p; best_cost = cost; }
+    }
+    if (best == 1 || best_cost * 100 > 92 * whole_cost) return w;
+    w.split = best; w.rem = (int)rem; w.whole = tiles - rem; w.items = w.whole + rem * best;
+    return w;
 }
 
 // Prefix sums of rows and m-tiles over the experts, built by the first wavefront
@@ -122,26 +170,27 @@ struct TileCoord {
     int rows_e;   // rows of the expert from row0 on (>= 1; the tile holds min(rows_e, BM) of them)
 };
 
-// Work item q -> tile.  Items are cut in rounds of G (the grid size); inside a round, item q belongs to XCD
-// q % 8 and the XCD's items of the round are consecutive tiles.  Inside an expert the tiles are ordered in
-// bands of 4 m-tiles (a lone fifth, ninth, ... m-tile joins the band before it); a band walks the n-tiles
-// with its m-tiles innermost, so a weight tile is shared by the band's m-tiles on one L2 and the band's A
-// rows stay there while it sweeps N.
+// Work item q -> position L in the tile order.  Items are cut in rounds of G (the grid size); inside a round, item q
+// belongs to XCD q % 8 and the XCD's items of the round are consecutive positions.
+__device__ __forceinline__ long long item_order(long long q, int G, long long total) {
+    if (G % kXcds != 0) return q;
+    // a round holds cnt = min(G, items left) items; XCD x owns those with q % 8 == x, cnt / 8 of them plus one
+    // more on the first cnt % 8 XCDs, and they map onto consecutive positions (a bijection for every cnt, so the
+    // last, partly filled round - the only round of a small problem - keeps its operand sharing too)
+    const long long base = (q / G) * G;
+    const long long left = total - base;
+    const int cnt = (int)(left < G ? left : G);
+    const int w = (int)(q - base), x = w % kXcds;
+    const int per = cnt / kXcds, extra = cnt % kXcds;
+    return base + (long long)x * per + (x < extra ? x : extra) + (w / kXcds);
+}
+
+// Position L in the tile order -> tile.  Inside an expert the tiles are ordered in bands of 4 m-tiles (a lone fifth,
+// ninth, ... m-tile joins the band before it); a band walks the n-tiles with its m-tiles innermost, so a weight tile
+// is shared by the band's m-tiles on one L2 and the band's A rows stay there while it sweeps N.
 template <int BM>
-__device__ __forceinline__ TileCoord decode_tile(long long q, int G, long long total, int n_tiles, int E,
-                                                 const int *s_tile_start, const int *s_row_start) {
-    long long L = q;
-    if (G % kXcds == 0) {
-        // a round holds cnt = min(G, items left) items; XCD x owns those with q % 8 == x, cnt / 8 of them plus one
-        // more on the first cnt % 8 XCDs, and they map onto consecutive tiles (a bijection for every cnt, so the
-        // last, partly filled round - the only round of a small problem - keeps its operand sharing too)
-        const long long base = (q / G) * G;
-        const long long left = total - base;
-        const int cnt = (int)(left < G ? left : G);
-        const int w = (int)(q - base), x = w % kXcds;
-        const int per = cnt / kXcds, extra = cnt % kXcds;
-        L = base + (long long)x * per + (x < extra ? x : extra) + (w / kXcds);
-    }
+__device__ __forceinline__ TileCoord decode_tile(long long L, int n_tiles, int E, const int *s_tile_start,
+                                                 const int *s_row_start) {
     const int u = (int)(L / n_tiles);
     int lo = 0, hi = E;  // last e with s_tile_start[e] <= u
     while (hi - lo > 1) {
@@ -169,7 +218,33 @@ __device__ __forceinline__ TileCoord decode_tile(long long q, int G, long long t
     return t;
 }
 
-int next_sched_slot();
+// A work item: a tile and the stages [s_lo, s_lo + s_cnt) of it; piece >= 0 numbers the piece of a split tile,
+// whose number among the split tiles is `split_tile`.
+struct WorkItem {
+    TileCoord tile;
+    int s_lo, s_cnt;
+    int piece;
+    int split_tile;
+};
+template <int BM>
+__device__ __forceinline__ WorkItem decode_item(long long q, int G, const WorkPlan &w, int stages, int n_tiles, int E,
+                                                const int *s_tile_start, const int *s_row_start) {
+    const long long L = item_order(q, G, w.items);
+    WorkItem it;
+    long long tile = L;
+    it.s_lo = 0; it.s_cnt = stages; it.piece = -1; it.split_tile = 0;
+    if (L >= w.whole) {
+        const long long r = L - w.whole;            // piece-major: the same piece of consecutive tiles is consecutive
+        it.piece = (int)(r / w.rem);
+        it.split_tile = (int)(r - (long long)it.piece * w.rem);
+        tile = w.whole + it.split_tile;
+        it.s_lo = (int)((long long)stages * it.piece / w.split);
+        it.s_cnt = (int)((long long)stages * (it.piece + 1) / w.split) - it.s_lo;
+    }
+    it.tile = decode_tile<BM>(tile, n_tiles, E, s_tile_start, s_row_start);
+    return it;
+}
+
 int launch_direct_bf16(const GmmArgs &args, int tile_rows, bool trans_b, bool swiglu, hipStream_t stream);
 int launch_direct_fp8(const GmmArgs &args, int tile_rows, bool swiglu, hipStream_t stream);
 

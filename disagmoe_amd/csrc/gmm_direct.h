@@ -71,7 +71,9 @@ constexpr int kStageB = kDN * kDK * 2;     // 16 KiB of B per stage
 // NP = 0: every wavefront copies its share of a stage and computes.  NP = 2: wavefronts NW and NW + 1 only copy
 // (and draw the work items), the first NW only compute: a copy that waits for room in the memory pipeline then holds
 // up no MFMA, which is what small tiles on weights streamed from HBM need.
-template <int kDM, int NW, int WM, bool TRANS_B, bool SWIGLU, bool FP8, int NP = 0>
+// PP = 1 (bf16 on 8 wavefronts): the two wavefronts of a SIMD alternate between a phase of operand reads and copies
+// and a phase of nothing but MFMAs, half a step apart, handed over by workgroup barriers.
+template <int kDM, int NW, int WM, bool TRANS_B, bool SWIGLU, bool FP8, int NP = 0, int PP = 0>
 __global__ __launch_bounds__((NW + NP) * 64) __attribute__((amdgpu_waves_per_eu((NW + NP + 3) / 4, (NW + NP + 3) / 4)))
 void gmm_direct_kernel(const GmmArgs p) {
     constexpr int kStageK = FP8 ? 64 : kDK;               // k per stage: 64 bytes per row either way
@@ -94,6 +96,7 @@ void gmm_direct_kernel(const GmmArgs p) {
     static_assert((NW == 4 || NW == 8) && WM * WN == NW && CA >= 1 && FM >= 1 && FN >= 2 && NR <= NM, "wave layout");
     static_assert(NP == 0 || (NP == 2 && NW == 4 && !FP8), "copying wavefronts: two, beside four computing ones");
     static_assert((kStages - 1) * kLoads <= 63, "vmcnt is a 6-bit counter");
+    static_assert(PP == 0 || (NW == 8 && WM == 2 && NP == 0 && !FP8 && kLoads % 2 == 0), "alternating phases: bf16 on 8 wavefronts");
     extern __shared__ __attribute__((aligned(16))) char smem[];
     __shared__ int s_tile_start[kMaxGroups + 1];
     __shared__ int s_row_start[kMaxGroups + 1];
@@ -110,9 +113,13 @@ void gmm_direct_kernel(const GmmArgs p) {
 
     const int n_out = SWIGLU ? p.N / 2 : p.N;
     const int n_tiles = (n_out + BNO - 1) / BNO;
-    const long long total = (long long)s_tile_start[E] * n_tiles;
-    const int S = p.K / kStageK;                   // stages (whole stages only)
+    const int S_all = p.K / kStageK;               // stages of a whole tile (whole stages only)
     const int G = gridDim.x;
+    // tiles of the last, partly filled round are cut along K (plan_work) when the launch has a workspace for their sums
+    constexpr long long kPieceBytes = (long long)kDM * kDN * sizeof(float);
+    const WorkPlan plan = plan_work((long long)s_tile_start[E] * n_tiles, G, S_all,
+                                    p.arrive != nullptr ? p.partial_bytes / kPieceBytes : 0, kWsArriveCount / NW);
+    const long long total = plan.items;
     const uint32_t pitch = (uint32_t)p.K * (FP8 ? 1 : 2);   // bytes per row of a (and of b when K-contiguous)
     const uint32_t smem_addr = lds_addr(smem);
 
@@ -135,6 +142,8 @@ void gmm_direct_kernel(const GmmArgs p) {
 
     // ---- state of the tile whose copies are being issued (set by open_tile) ----
     int e = 0, row0 = 0, rows_e = 0, n0 = 0;
+    int s_lo = 0, S = 0, pre = 0;        // its stages [s_lo, s_lo + S); pre = the first of them, copied ahead of its first MFMA
+    int part = -1, split_tile = 0;       // piece of a split tile (-1: a whole tile) and the tile's number among those
     uint64_t a_base = 0, b_exp = 0;      // wave-uniform bases of the tile's rows of a and of the expert's weights
     uint32_t a_off[CA], b_off[CB];        // per-lane byte offsets of this wavefront's copies from those bases
 
@@ -146,13 +155,17 @@ void gmm_direct_kernel(const GmmArgs p) {
         return base + (rh < n_out - n0 ? rh : 0);
     };
     auto locate_tile = [&](long long q) {
-        const TileCoord tc = decode_tile<kDM>(q, G, total, n_tiles, E, s_tile_start, s_row_start);
-        e = tc.e; row0 = tc.row0; rows_e = tc.rows_e; n0 = tc.nt * BNO;
+        const WorkItem it = decode_item<kDM>(q, G, plan, S_all, n_tiles, E, s_tile_start, s_row_start);
+        e = it.tile.e; row0 = it.tile.row0; rows_e = it.tile.rows_e; n0 = it.tile.nt * BNO;
+        s_lo = it.s_lo; S = it.s_cnt; pre = S < kStages ? S : kStages;
+        part = it.piece; split_tile = it.split_tile;
     };
     auto open_tile = [&](long long q) {
         locate_tile(q);
-        a_base = to_scalar((uint64_t)(uintptr_t)p.a + (uint64_t)row0 * pitch);
-        b_exp = to_scalar((uint64_t)(uintptr_t)p.b + (uint64_t)e * p.K * p.N * (FP8 ? 1 : 2));
+        // stage s of the item is stage s_lo + s of the tile
+        a_base = to_scalar((uint64_t)(uintptr_t)p.a + (uint64_t)row0 * pitch + (uint64_t)s_lo * 64);
+        b_exp = to_scalar((uint64_t)(uintptr_t)p.b + (uint64_t)e * p.K * p.N * (FP8 ? 1 : 2) +
+                          (uint64_t)s_lo * (TRANS_B ? 64 : (uint64_t)kDK * p.N * 2));
 #pragma unroll
         for (int i = 0; i < CA; ++i) {
             int r = (i * NC + cw) * 16 + kc_row;
@@ -182,7 +195,6 @@ void gmm_direct_kernel(const GmmArgs p) {
             else copy_g2lds_16<kStageA + i * kBlock>(b_off[i], b_exp + (uint64_t)s * kDK * p.N * 2, lds);
         }
     };
-    const int pre = S < kStages ? S : kStages;      // stages whose copies are issued ahead of the tile's first MFMA
     auto issue_prologue = [&]() {
         for (int s = 0; s < pre; ++s) {
             static_for<0, kLoads>([&](auto c) { issue_copy(s, c); });
@@ -256,9 +268,9 @@ void gmm_direct_kernel(const GmmArgs p) {
     unsigned int draw = 0;
     const bool drawer = tid == (NP ? NW * 64 : 0);
     if (drawer) {
-        draw = sched_draw(p.sched_slot, streams);
+        draw = sched_draw(p.sched, streams);
         s_item = sched_item(draw, streams);
-        draw = sched_draw(p.sched_slot, streams);   // always one draw ahead: its round trip hides behind a tile
+        draw = sched_draw(p.sched, streams);   // always one draw ahead: its round trip hides behind a tile
     }
     __syncthreads();
     long long q = s_item;
@@ -287,12 +299,12 @@ void gmm_direct_kernel(const GmmArgs p) {
                 __syncthreads();                   // the last stage has been read: all of the LDS may be refilled
                 q = s_item;
                 if (q < total) {
-                    if (drawer) draw = sched_draw(p.sched_slot, streams);
+                    if (drawer) draw = sched_draw(p.sched, streams);
                     open_tile(q);
                     issue_prologue();
                 }
             }
-            sched_finish(p.sched_slot);
+            sched_finish(p.sched);
             return;
         }
     }
@@ -300,6 +312,7 @@ void gmm_direct_kernel(const GmmArgs p) {
     while (q < total) {
         // results of this tile go here after the next tile's copies have been issued
         const int cur_row0 = row0, cur_rows_e = rows_e, cur_n0 = n0, cur_e = e;
+        const int cur_part = part, cur_split_tile = split_tile;
         // row fragments of this wavefront that hold at least one valid row (a short last tile skips the rest)
         int nfr = ((rows_e < kDM ? rows_e : kDM) - wm * TM + 31) / 32;
         nfr = __builtin_amdgcn_readfirstlane(nfr < 0 ? 0 : (nfr > FM ? FM : nfr));
@@ -333,6 +346,50 @@ void gmm_direct_kernel(const GmmArgs p) {
         // epilogue that were issued after them, may still be in flight: waiting for fewer is only stricter)
         if constexpr (NP == 0) wait_ahead(pre - 1);
         __syncthreads();
+        if constexpr (PP != 0) {
+            // Alternating phases.  A k-step is a memory phase (the NR operand reads of the step into the one register
+            // set, this wavefront's copies, the waits) and a matrix phase (the NM MFMAs, nothing else), each closed
+            // by a workgroup barrier.  The wavefronts of the lower half of the tile (wm == 1) run one phase behind the
+            // others, and wavefronts w and w + 4 share a SIMD: while one of them issues MFMAs the other one issues
+            // everything else.  The slot of stage s - 1 is free once every wavefront has read k-step 1 of that stage,
+            // i.e. behind the barrier that closes the memory phase of the late half; from then on (memory phases of
+            // stage s) it is refilled with stage s + kStages - 1.
+            // (A phase per stage - twice the MFMAs, a register set per k-step, half the barriers - is no faster.)
+            auto pp_stage = [&](int s, auto refill_tag, int ahead, bool next) {
+                constexpr bool kRefill = decltype(refill_tag)::value;
+                auto landed = [&]() {   // this wavefront's copies of stage s + 1 have landed
+                    if constexpr (kRefill) DMOE_WAIT_VMCNT((kStages - 2) * kLoads);
+                    else wait_ahead(ahead);
+                };
+                static_for<0, 2>([&](auto ks_tag) {
+                    constexpr int ks = decltype(ks_tag)::value;
+#pragma unroll
+                    for (int r = 0; r < NR; ++r) load_frag(s, ks, 0, r);
+                    if constexpr (kRefill)
+                        static_for<ks * kLoads / 2, (ks + 1) * kLoads / 2>([&](auto c) { issue_copy(s + kStages - 1, c); });
+                    if (ks == 1 && next && wm == 1) landed();
+                    __builtin_amdgcn_sched_barrier(0);
+                    __syncthreads();
+                    __builtin_amdgcn_sched_barrier(0);
+                    __builtin_amdgcn_s_setprio(1);
+                    static_for<0, NM>([&](auto t_tag) { mfma_one(0, decltype(t_tag)::value); });
+                    __builtin_amdgcn_s_setprio(0);
+                    if (ks == 1 && next && wm == 0) landed();
+                    __builtin_amdgcn_sched_barrier(0);
+                    __syncthreads();
+                    __builtin_amdgcn_sched_barrier(0);
+                });
+            };
+            if (wm == 1) __syncthreads();
+            int s = 0;
+            pp_stage(0, std::false_type{}, (S - 2 < kStages - 2 ? S - 2 : kStages - 2), S > 1);
+            for (s = 1; s + kStages - 1 < S; ++s) pp_stage(s, std::true_type{}, 0, true);
+            for (; s < S; ++s) {
+                const int left = S - 1 - s;
+                pp_stage(s, std::false_type{}, left - 1 < kStages - 2 ? left - 1 : kStages - 2, left > 0);
+            }
+            if (wm == 0) __syncthreads();
+        } else {
 #pragma unroll
         for (int r = 0; r < NR; ++r) load_frag(0, 0, 0, r);
 
@@ -428,6 +485,7 @@ void gmm_direct_kernel(const GmmArgs p) {
             step(s, std::false_type{}, left - 1 < kStages - 2 ? left - 1 : kStages - 2, left > 0,
                  !FP8 && s > 0 && s + kStages == S);
         }
+        }   // PP == 0
 
         if constexpr (NP > 0) {
             __syncthreads();   // every wavefront has read its last fragments: the copying wavefronts may refill the LDS
@@ -556,9 +614,62 @@ void gmm_direct_kernel(const GmmArgs p) {
                     }
                 }
             }
-    
         };
-        epilogue();
+        bool finish = true;
+        if (cur_part >= 0) {
+            // ---- a piece of a split tile ----
+            // Every wavefront leaves its accumulators in the workspace, as [fragment][4 values][lane] so that an
+            // instruction moves 1 KiB, and counts itself in at the counter of its part of the tile.  The wavefront that
+            // arrives last there, of whichever piece, adds the pieces up in their order and goes on to the epilogue.
+            // The partial sums and the counter are written and read with accesses of device scope, which go past the
+            // XCD's L2 to memory that every XCD sees: no fence has to write back or invalidate a whole L2, whose
+            // other contents (the operand tiles of the compute units beside this one) stay where they are.
+            constexpr int kWaveFloats = TM * TN;
+            unsigned long long *mine = (unsigned long long *)(p.partials + ((size_t)(cur_split_tile * plan.split + cur_part) * NW + wave) * kWaveFloats);
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+#pragma unroll
+                for (int j = 0; j < FN; ++j)
+#pragma unroll
+                    for (int x = 0; x < 8; ++x) {
+                        const unsigned long long v = (unsigned long long)__float_as_uint(acc[i][j][2 * x]) |
+                                                     ((unsigned long long)__float_as_uint(acc[i][j][2 * x + 1]) << 32);
+                        __hip_atomic_store(mine + ((i * FN + j) * 8 + x) * 64 + lane, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+            // the stores have reached memory before the wavefront counts itself in
+            __atomic_signal_fence(__ATOMIC_SEQ_CST);
+            DMOE_WAIT_VMCNT(0);
+            __atomic_signal_fence(__ATOMIC_SEQ_CST);
+            unsigned int *arrived = p.arrive + cur_split_tile * NW + wave;
+            unsigned int before = 0;
+            if (lane == 0) before = __hip_atomic_fetch_add(arrived, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            before = __builtin_amdgcn_readfirstlane(before);
+            __atomic_signal_fence(__ATOMIC_SEQ_CST);
+            finish = before == (unsigned int)(plan.split - 1);
+            if (finish) {
+                if (lane == 0) __hip_atomic_store(arrived, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // as the next launch expects it
+#pragma unroll
+                for (int i = 0; i < FM; ++i)
+#pragma unroll
+                    for (int j = 0; j < FN; ++j)
+#pragma unroll
+                        for (int x = 0; x < 16; ++x) acc[i][j][x] = 0.f;
+                for (int k = 0; k < plan.split; ++k) {
+                    unsigned long long *src = (unsigned long long *)(p.partials + ((size_t)(cur_split_tile * plan.split + k) * NW + wave) * kWaveFloats);
+#pragma unroll
+                    for (int i = 0; i < FM; ++i)
+#pragma unroll
+                        for (int j = 0; j < FN; ++j)
+#pragma unroll
+                            for (int x = 0; x < 8; ++x) {
+                                const unsigned long long v = __hip_atomic_load(src + ((i * FN + j) * 8 + x) * 64 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                                acc[i][j][2 * x] += __uint_as_float((unsigned int)v);
+                                acc[i][j][2 * x + 1] += __uint_as_float((unsigned int)(v >> 32));
+                            }
+                }
+            }
+        }
+        if (finish) epilogue();
         };   // run_tile
         // fp8: one instance per wavefront number (the MFMA slots of its copies are compile-time constants)
         auto run_build = [&](auto guard_tag) {
@@ -584,7 +695,7 @@ void gmm_direct_kernel(const GmmArgs p) {
             __syncthreads();   // also: the last stage has been read by everyone, LDS may be refilled
             q = s_item;
             if (q < total) {
-                if (drawer) draw = sched_draw(p.sched_slot, streams);
+                if (drawer) draw = sched_draw(p.sched, streams);
                 open_tile(q);
                 issue_prologue();
             }
@@ -593,15 +704,15 @@ void gmm_direct_kernel(const GmmArgs p) {
         if constexpr (NP == 0) next_item();
         else if (q < total) locate_tile(q);
     }
-    sched_finish(p.sched_slot);
+    sched_finish(p.sched);
 }
 
-template <int kDM, int NW, int WM, bool TRANS_B, bool SWIGLU, bool FP8, int NP = 0>
+template <int kDM, int NW, int WM, bool TRANS_B, bool SWIGLU, bool FP8, int NP = 0, int PP = 0>
 static int launch_direct_one(const GmmArgs &args, hipStream_t stream) {
     constexpr int BNO = SWIGLU ? kDN / 2 : kDN;
     constexpr int kStages = kDM == 256 ? 4 : (kDM == 128 ? 5 : 6);
     const size_t lds = (size_t)kStages * (kDM * kDK * 2 + kStageB);
-    auto kern = gmm_direct_kernel<kDM, NW, WM, TRANS_B, SWIGLU, FP8, NP>;
+    auto kern = gmm_direct_kernel<kDM, NW, WM, TRANS_B, SWIGLU, FP8, NP, PP>;
     static unsigned long long configured = 0;   // devices on which the kernel's LDS size has been raised
     DMOE_HIP(raise_dynamic_lds((const void *)kern, (int)lds, &configured));
     const int n_out = SWIGLU ? args.N / 2 : args.N;
@@ -611,17 +722,15 @@ static int launch_direct_one(const GmmArgs &args, hipStream_t stream) {
     if (m_tiles_max * n_tiles < grid) grid = m_tiles_max * n_tiles;
     if (grid < 1) grid = 1;
     grid = (grid + kXcds - 1) / kXcds * kXcds;   // whole rows of XCDs: the tile order is XCD-aware only then
-    GmmArgs launch_args = args;
-    launch_args.sched_slot = next_sched_slot();
-    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3((NW + NP) * 64), lds, stream, launch_args);
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3((NW + NP) * 64), lds, stream, args);
     DMOE_LAUNCH_CHECK("gmm_direct_kernel");
     return DMOE_OK;
 }
 
-template <int kDM, int NW, int WM, int NP = 0>
+template <int kDM, int NW, int WM, int NP = 0, int PP = 0>
 static int launch_direct_tile(const GmmArgs &args, bool trans_b, bool swiglu, hipStream_t stream) {
-    if (trans_b) return swiglu ? launch_direct_one<kDM, NW, WM, true, true, false, NP>(args, stream) : launch_direct_one<kDM, NW, WM, true, false, false, NP>(args, stream);
-    return swiglu ? launch_direct_one<kDM, NW, WM, false, true, false, NP>(args, stream) : launch_direct_one<kDM, NW, WM, false, false, false, NP>(args, stream);
+    if (trans_b) return swiglu ? launch_direct_one<kDM, NW, WM, true, true, false, NP, PP>(args, stream) : launch_direct_one<kDM, NW, WM, true, false, false, NP, PP>(args, stream);
+    return swiglu ? launch_direct_one<kDM, NW, WM, false, true, false, NP, PP>(args, stream) : launch_direct_one<kDM, NW, WM, false, false, false, NP, PP>(args, stream);
 }
 
 }  // namespace dmoe

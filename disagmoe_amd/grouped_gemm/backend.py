@@ -24,6 +24,59 @@ def _sizes_on_device(batch_sizes: torch.Tensor, device: torch.device) -> torch.T
     return batch_sizes.to(device=device, dtype=torch.int64, non_blocking=True).contiguous()
 
 
+# ---- state blocks and workspaces ---------------------------------------------
+# A launch keeps its work counters in a zeroed state block and the partial sums of
+# the tiles it cuts along K in a workspace (include/dmoe.h).  ``get_arguments``
+# hands out a state block (its address is the ``arguments_ptr`` of the reference's
+# API) and the caller allocates the workspace, as experts.py:69-77 does; calls
+# without them use a pair that this module keeps per device and stream.
+
+_STATE_BLOCKS = {}     # address -> the zeroed uint8 tensor behind an arguments_ptr
+_DEFAULTS = {}         # (device index, stream handle) -> (state block, workspace)
+
+
+def workspace_bytes(num_experts: int = 1) -> int:
+    """Size of the workspace at which no launch is short of room (dmoe_gmm_workspace_bytes)."""
+    need = _lib.c_size_t(0)
+    _lib.call("dmoe_gmm_workspace_bytes", int(num_experts), _lib.ctypes.byref(need))
+    return int(need.value)
+
+
+def _new_state_block(device: torch.device) -> torch.Tensor:
+    return torch.zeros(_lib.GMM_STATE_BYTES, dtype=torch.uint8, device=device)
+
+
+def _default_state(device: torch.device, stream: int):
+    """``(state block address, workspace address, workspace bytes)`` of stream ``stream`` of
+    ``device``: launches on one stream never overlap, so they can share the pair."""
+    key = (device.index, stream)
+    pair = _DEFAULTS.get(key)
+    if pair is None:
+        with torch.cuda.device(device):
+            state, ws = _new_state_block(device), torch.empty(workspace_bytes(), dtype=torch.uint8, device=device)
+        pair = (state.data_ptr(), ws.data_ptr(), ws.numel(), state, ws)    # the tensors keep the memory alive
+        _DEFAULTS[key] = pair
+    return pair[:3]
+
+
+def _state_args(device: torch.device, workspace: Optional[torch.Tensor], arguments_ptr: Optional[int], stream: int):
+    """The three state arguments of a dmoe_gmm* call and its stream."""
+    return (*_state_triple(device, workspace, arguments_ptr, stream), stream)
+
+
+def _state_triple(device, workspace, arguments_ptr, stream):
+    if arguments_ptr is None and workspace is None:
+        return _default_state(device, stream)
+    if not arguments_ptr:
+        raise ValueError("a caller-owned workspace needs the arguments_ptr that get_arguments returned with its size")
+    if arguments_ptr not in _STATE_BLOCKS:
+        raise ValueError(f"arguments_ptr {arguments_ptr:#x} does not come from get_arguments")
+    if workspace is None:
+        return arguments_ptr, None, 0
+    assert workspace.dtype == torch.uint8 and workspace.is_contiguous() and workspace.device == device
+    return arguments_ptr, workspace.data_ptr(), workspace.numel()
+
+
 def _check_operands(a: torch.Tensor, b: torch.Tensor, dtype: torch.dtype) -> torch.device:
     if not a.is_cuda:
         raise RuntimeError("gmm needs device tensors; disagmoe_amd has no CPU fallback")
@@ -35,11 +88,14 @@ def _check_operands(a: torch.Tensor, b: torch.Tensor, dtype: torch.dtype) -> tor
 
 
 def gmm(a: torch.Tensor, b: torch.Tensor, batch_sizes: torch.Tensor, trans_b: bool = False,
-        c: Optional[torch.Tensor] = None) -> torch.Tensor:
+        c: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None,
+        arguments_ptr: Optional[int] = None) -> torch.Tensor:
     """``c[o_e:o_e+n_e] = a[o_e:o_e+n_e] @ b[e]`` (``b[e].T`` with ``trans_b``),
     bf16 operands, fp32 accumulation, bf16 result.  ``c`` (optional) is a
     preallocated ``[>= rows, N]`` buffer written in place and returned
-    (experts.py:84,89); rows past ``sum(batch_sizes)`` are left untouched."""
+    (experts.py:84,89); rows past ``sum(batch_sizes)`` are left untouched.
+    ``workspace``/``arguments_ptr`` as :func:`gmm_with_arguments` takes them;
+    without them the call uses the pair this module keeps for the current stream."""
     device = _check_operands(a, b, torch.bfloat16)
     rows, K = a.shape
     E = b.shape[0]
@@ -54,12 +110,13 @@ def gmm(a: torch.Tensor, b: torch.Tensor, batch_sizes: torch.Tensor, trans_b: bo
     bs = _sizes_on_device(batch_sizes, device)
     with torch.cuda.device(device):
         _lib.call("dmoe_gmm", a.data_ptr(), b.data_ptr(), c.data_ptr(), bs.data_ptr(), rows, E, K, N,
-                  1 if trans_b else 0, _lib.BF16, _stream(device))
+                  1 if trans_b else 0, _lib.BF16, *_state_args(device, workspace, arguments_ptr, _stream(device)))
     return c
 
 
 def gmm_swiglu(a: torch.Tensor, b: torch.Tensor, batch_sizes: torch.Tensor, trans_b: bool = False,
-               c: Optional[torch.Tensor] = None) -> torch.Tensor:
+               c: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None,
+               arguments_ptr: Optional[int] = None) -> torch.Tensor:
     """Gate-up projection with the activation fused: ``silu(u[:, :I]) * u[:, I:]``
     for ``u = gmm(a, b)``, ``b [E, K, 2I]`` (``[E, 2I, K]`` with ``trans_b``);
     returns ``[rows, I]``.  The two steps of experts.py:92-93 in one kernel, taken
@@ -78,27 +135,33 @@ def gmm_swiglu(a: torch.Tensor, b: torch.Tensor, batch_sizes: torch.Tensor, tran
     bs = _sizes_on_device(batch_sizes, device)
     with torch.cuda.device(device):
         _lib.call("dmoe_gmm_swiglu", a.data_ptr(), b.data_ptr(), c.data_ptr(), bs.data_ptr(), rows, E, K, inter,
-                  1 if trans_b else 0, _lib.BF16, _stream(device))
+                  1 if trans_b else 0, _lib.BF16, *_state_args(device, workspace, arguments_ptr, _stream(device)))
     return c
 
 
 def get_arguments(num_experts: int, device: torch.device) -> Tuple[int, int]:
-    """``(workspace_size, arguments_ptr)`` as in experts.py:69-72.  The HIP
-    scheduler builds its work list on the device inside the kernel, so the
-    workspace is a token allocation and the handle is 0."""
-    need = _lib.c_size_t(0)
-    _lib.call("dmoe_gmm_workspace_bytes", int(num_experts), _lib.ctypes.byref(need))
-    return int(need.value), 0
+    """``(workspace_size, arguments_ptr)`` as in experts.py:69-72 and
+    tests/ops/test_gemm.py:24.  ``arguments_ptr`` is the address of a zeroed state
+    block on ``device`` that this module keeps alive (the launch's work counters
+    live there); ``workspace_size`` is the size of the buffer the caller allocates
+    (``torch.empty``, any contents) for the partial sums of tiles cut along K."""
+    device = torch.device(device)
+    if device.type != "cuda":
+        raise RuntimeError("get_arguments needs a HIP device; disagmoe_amd has no CPU fallback")
+    with torch.cuda.device(device):
+        block = _new_state_block(device)
+    _STATE_BLOCKS[block.data_ptr()] = block
+    return workspace_bytes(num_experts), block.data_ptr()
 
 
 def gmm_with_arguments(a: torch.Tensor, b: torch.Tensor, batch_sizes: torch.Tensor, workspace: torch.Tensor,
                        arguments_ptr: int, **kwargs) -> torch.Tensor:
-    """Same result as :func:`gmm`, bit for bit, with a caller-owned workspace
-    (experts.py:74-77; tests/ops/test_gemm.py:30-36 call it repeatedly with one
-    workspace).  Neither form allocates scheduler state on the host."""
-    size, _ = get_arguments(b.shape[0], a.device)
-    assert workspace.dtype == torch.uint8 and workspace.numel() >= size
-    return gmm(a, b, batch_sizes, **kwargs)
+    """:func:`gmm` with the caller's workspace and the state block behind
+    ``arguments_ptr`` (experts.py:74-77; tests/ops/test_gemm.py:30-36 call it
+    repeatedly with one pair).  Same result as :func:`gmm`, bit for bit, for a
+    workspace of the size ``get_arguments`` stated; nothing is allocated."""
+    assert workspace.dtype == torch.uint8
+    return gmm(a, b, batch_sizes, workspace=workspace, arguments_ptr=arguments_ptr, **kwargs)
 
 
 # ---- fp8 (e4m3fn) forms: no counterpart in the reference --------------------
@@ -144,7 +207,8 @@ def _fp8_common(a, a_scale, b, b_scale):
 
 
 def gmm_fp8(a: torch.Tensor, a_scale: torch.Tensor, b: torch.Tensor, b_scale: torch.Tensor,
-            batch_sizes: torch.Tensor, c: Optional[torch.Tensor] = None) -> torch.Tensor:
+            batch_sizes: torch.Tensor, c: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None,
+            arguments_ptr: Optional[int] = None) -> torch.Tensor:
     """``c = (a @ b[e].T) * a_scale[:, None] * b_scale[e][None, :]`` in bf16; ``a``
     fp8 ``[rows, K]``, ``b`` fp8 ``[E, N, K]``."""
     rows, K, E, N = _fp8_common(a, a_scale, b, b_scale)
@@ -153,12 +217,13 @@ def gmm_fp8(a: torch.Tensor, a_scale: torch.Tensor, b: torch.Tensor, b_scale: to
     bs = _sizes_on_device(batch_sizes, a.device)
     with torch.cuda.device(a.device):
         _lib.call("dmoe_gmm_fp8", a.data_ptr(), a_scale.data_ptr(), b.data_ptr(), b_scale.data_ptr(), c.data_ptr(),
-                  bs.data_ptr(), rows, E, K, N, _stream(a.device))
+                  bs.data_ptr(), rows, E, K, N, *_state_args(a.device, workspace, arguments_ptr, _stream(a.device)))
     return c
 
 
 def gmm_fp8_swiglu(a: torch.Tensor, a_scale: torch.Tensor, b: torch.Tensor, b_scale: torch.Tensor,
-                   batch_sizes: torch.Tensor, c: Optional[torch.Tensor] = None) -> torch.Tensor:
+                   batch_sizes: torch.Tensor, c: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None,
+                   arguments_ptr: Optional[int] = None) -> torch.Tensor:
     """fp8 gate-up projection with fused ``silu(gate) * up``; ``b`` fp8 ``[E, 2I,
     K]``; returns bf16 ``[rows, I]``."""
     rows, K, E, N2 = _fp8_common(a, a_scale, b, b_scale)
@@ -168,7 +233,7 @@ def gmm_fp8_swiglu(a: torch.Tensor, a_scale: torch.Tensor, b: torch.Tensor, b_sc
     bs = _sizes_on_device(batch_sizes, a.device)
     with torch.cuda.device(a.device):
         _lib.call("dmoe_gmm_fp8_swiglu", a.data_ptr(), a_scale.data_ptr(), b.data_ptr(), b_scale.data_ptr(),
-                  c.data_ptr(), bs.data_ptr(), rows, E, K, N2 // 2, _stream(a.device))
+                  c.data_ptr(), bs.data_ptr(), rows, E, K, N2 // 2, *_state_args(a.device, workspace, arguments_ptr, _stream(a.device)))
     return c
 
 

@@ -58,20 +58,22 @@ class MoEExperts(torch.nn.Module):
         self.cache_up = torch.empty((max_batch_size, self.intermediate_size), dtype=params_dtype, device=dev)
         self.cache_down = torch.empty((max_batch_size, self.hidden_size), dtype=params_dtype, device=dev)
         self.enable_cache = enable_cutlass_cache
-        if enable_cutlass_cache:
-            self.workspace_size, self.arguments_ptr = gg.get_arguments(self.num_experts, dev)
-            self.workspace = torch.empty([self.workspace_size], dtype=torch.uint8, device=dev)
+        # state block and workspace of this layer's launches (experts.py:69-77): a captured graph of the layer then
+        # shares its scheduler state with no other launch
+        self.workspace_size, self.arguments_ptr = gg.get_arguments(self.num_experts, dev)
+        self.workspace = torch.empty([self.workspace_size], dtype=torch.uint8, device=dev)
 
     def forward(self, bs: int, hiddens: torch.Tensor, batch_sizes: torch.Tensor) -> torch.Tensor:
         """``gmm(silu(u[:, :I]) * u[:, I:], w2)`` with ``u = gmm(hiddens, w13)``
         (experts.py:92-96); gate-up, SiLU and the product are one kernel.  Below
         ``max_batch_size`` rows the static buffers are used (the reference's
         cached branch, :83-90)."""
+        ws = dict(workspace=getattr(self, "workspace", None), arguments_ptr=getattr(self, "arguments_ptr", None))
         if self.enable_cache and bs <= self.gmm_cache_max_batch_size and hiddens.shape[0] <= self.cache_up.shape[0]:
-            h = gg.gmm_swiglu(hiddens, self.w13_weight, batch_sizes, c=self.cache_up)[:hiddens.shape[0]]
-            return gg.gmm(h, self.w2_weight, batch_sizes, c=self.cache_down)[:hiddens.shape[0]]
-        h = gg.gmm_swiglu(hiddens, self.w13_weight, batch_sizes)
-        return gg.gmm(h, self.w2_weight, batch_sizes)
+            h = gg.gmm_swiglu(hiddens, self.w13_weight, batch_sizes, c=self.cache_up, **ws)[:hiddens.shape[0]]
+            return gg.gmm(h, self.w2_weight, batch_sizes, c=self.cache_down, **ws)[:hiddens.shape[0]]
+        h = gg.gmm_swiglu(hiddens, self.w13_weight, batch_sizes, **ws)
+        return gg.gmm(h, self.w2_weight, batch_sizes, **ws)
 
     def forward_unfused(self, bs: int, hiddens: torch.Tensor, batch_sizes: torch.Tensor) -> torch.Tensor:
         """The reference's own schedule, statement by statement (experts.py:92-94):

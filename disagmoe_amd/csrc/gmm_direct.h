@@ -71,9 +71,7 @@ constexpr int kStageB = kDN * kDK * 2;     // 16 KiB of B per stage
 // NP = 0: every wavefront copies its share of a stage and computes.  NP = 2: wavefronts NW and NW + 1 only copy
 // (and draw the work items), the first NW only compute: a copy that waits for room in the memory pipeline then holds
 // up no MFMA, which is what small tiles on weights streamed from HBM need.
-// PP = 1 (bf16 on 8 wavefronts): the two wavefronts of a SIMD alternate between a phase of operand reads and copies
-// and a phase of nothing but MFMAs, half a step apart, handed over by workgroup barriers.
-template <int kDM, int NW, int WM, bool TRANS_B, bool SWIGLU, bool FP8, int NP = 0, int PP = 0>
+template <int kDM, int NW, int WM, bool TRANS_B, bool SWIGLU, bool FP8, int NP = 0>
 __global__ __launch_bounds__((NW + NP) * 64) __attribute__((amdgpu_waves_per_eu((NW + NP + 3) / 4, (NW + NP + 3) / 4)))
 void gmm_direct_kernel(const GmmArgs p) {
     constexpr int kStageK = FP8 ? 64 : kDK;               // k per stage: 64 bytes per row either way
@@ -96,7 +94,6 @@ void gmm_direct_kernel(const GmmArgs p) {
     static_assert((NW == 4 || NW == 8) && WM * WN == NW && CA >= 1 && FM >= 1 && FN >= 2 && NR <= NM, "wave layout");
     static_assert(NP == 0 || (NP == 2 && NW == 4 && !FP8), "copying wavefronts: two, beside four computing ones");
     static_assert((kStages - 1) * kLoads <= 63, "vmcnt is a 6-bit counter");
-    static_assert(PP == 0 || (NW == 8 && WM == 2 && NP == 0 && !FP8 && kLoads % 2 == 0), "alternating phases: bf16 on 8 wavefronts");
     extern __shared__ __attribute__((aligned(16))) char smem[];
     __shared__ int s_tile_start[kMaxGroups + 1];
     __shared__ int s_row_start[kMaxGroups + 1];
@@ -346,50 +343,6 @@ void gmm_direct_kernel(const GmmArgs p) {
         // epilogue that were issued after them, may still be in flight: waiting for fewer is only stricter)
         if constexpr (NP == 0) wait_ahead(pre - 1);
         __syncthreads();
-        if constexpr (PP != 0) {
-            // Alternating phases.  A k-step is a memory phase (the NR operand reads of the step into the one register
-            // set, this wavefront's copies, the waits) and a matrix phase (the NM MFMAs, nothing else), each closed
-            // by a workgroup barrier.  The wavefronts of the lower half of the tile (wm == 1) run one phase behind the
-            // others, and wavefronts w and w + 4 share a SIMD: while one of them issues MFMAs the other one issues
-            // everything else.  The slot of stage s - 1 is free once every wavefront has read k-step 1 of that stage,
-            // i.e. behind the barrier that closes the memory phase of the late half; from then on (memory phases of
-            // stage s) it is refilled with stage s + kStages - 1.
-            // (A phase per stage - twice the MFMAs, a register set per k-step, half the barriers - is no faster.)
-            auto pp_stage = [&](int s, auto refill_tag, int ahead, bool next) {
-                constexpr bool kRefill = decltype(refill_tag)::value;
-                auto landed = [&]() {   // this wavefront's copies of stage s + 1 have landed
-                    if constexpr (kRefill) DMOE_WAIT_VMCNT((kStages - 2) * kLoads);
-                    else wait_ahead(ahead);
-                };
-                static_for<0, 2>([&](auto ks_tag) {
-                    constexpr int ks = decltype(ks_tag)::value;
-#pragma unroll
-                    for (int r = 0; r < NR; ++r) load_frag(s, ks, 0, r);
-                    if constexpr (kRefill)
-                        static_for<ks * kLoads / 2, (ks + 1) * kLoads / 2>([&](auto c) { issue_copy(s + kStages - 1, c); });
-                    if (ks == 1 && next && wm == 1) landed();
-                    __builtin_amdgcn_sched_barrier(0);
-                    __syncthreads();
-                    __builtin_amdgcn_sched_barrier(0);
-                    __builtin_amdgcn_s_setprio(1);
-                    static_for<0, NM>([&](auto t_tag) { mfma_one(0, decltype(t_tag)::value); });
-                    __builtin_amdgcn_s_setprio(0);
-                    if (ks == 1 && next && wm == 0) landed();
-                    __builtin_amdgcn_sched_barrier(0);
-                    __syncthreads();
-                    __builtin_amdgcn_sched_barrier(0);
-                });
-            };
-            if (wm == 1) __syncthreads();
-            int s = 0;
-            pp_stage(0, std::false_type{}, (S - 2 < kStages - 2 ? S - 2 : kStages - 2), S > 1);
-            for (s = 1; s + kStages - 1 < S; ++s) pp_stage(s, std::true_type{}, 0, true);
-            for (; s < S; ++s) {
-                const int left = S - 1 - s;
-                pp_stage(s, std::false_type{}, left - 1 < kStages - 2 ? left - 1 : kStages - 2, left > 0);
-            }
-            if (wm == 0) __syncthreads();
-        } else {
 #pragma unroll
         for (int r = 0; r < NR; ++r) load_frag(0, 0, 0, r);
 
@@ -485,7 +438,6 @@ void gmm_direct_kernel(const GmmArgs p) {
             step(s, std::false_type{}, left - 1 < kStages - 2 ? left - 1 : kStages - 2, left > 0,
                  !FP8 && s > 0 && s + kStages == S);
         }
-        }   // PP == 0
 
         if constexpr (NP > 0) {
             __syncthreads();   // every wavefront has read its last fragments: the copying wavefronts may refill the LDS
@@ -707,12 +659,12 @@ void gmm_direct_kernel(const GmmArgs p) {
     sched_finish(p.sched);
 }
 
-template <int kDM, int NW, int WM, bool TRANS_B, bool SWIGLU, bool FP8, int NP = 0, int PP = 0>
+template <int kDM, int NW, int WM, bool TRANS_B, bool SWIGLU, bool FP8, int NP = 0>
 static int launch_direct_one(const GmmArgs &args, hipStream_t stream) {
     constexpr int BNO = SWIGLU ? kDN / 2 : kDN;
     constexpr int kStages = kDM == 256 ? 4 : (kDM == 128 ? 5 : 6);
     const size_t lds = (size_t)kStages * (kDM * kDK * 2 + kStageB);
-    auto kern = gmm_direct_kernel<kDM, NW, WM, TRANS_B, SWIGLU, FP8, NP, PP>;
+    auto kern = gmm_direct_kernel<kDM, NW, WM, TRANS_B, SWIGLU, FP8, NP>;
     static unsigned long long configured = 0;   // devices on which the kernel's LDS size has been raised
     DMOE_HIP(raise_dynamic_lds((const void *)kern, (int)lds, &configured));
     const int n_out = SWIGLU ? args.N / 2 : args.N;
@@ -727,10 +679,10 @@ static int launch_direct_one(const GmmArgs &args, hipStream_t stream) {
     return DMOE_OK;
 }
 
-template <int kDM, int NW, int WM, int NP = 0, int PP = 0>
+template <int kDM, int NW, int WM, int NP = 0>
 static int launch_direct_tile(const GmmArgs &args, bool trans_b, bool swiglu, hipStream_t stream) {
-    if (trans_b) return swiglu ? launch_direct_one<kDM, NW, WM, true, true, false, NP, PP>(args, stream) : launch_direct_one<kDM, NW, WM, true, false, false, NP, PP>(args, stream);
-    return swiglu ? launch_direct_one<kDM, NW, WM, false, true, false, NP, PP>(args, stream) : launch_direct_one<kDM, NW, WM, false, false, false, NP, PP>(args, stream);
+    if (trans_b) return swiglu ? launch_direct_one<kDM, NW, WM, true, true, false, NP>(args, stream) : launch_direct_one<kDM, NW, WM, true, false, false, NP>(args, stream);
+    return swiglu ? launch_direct_one<kDM, NW, WM, false, true, false, NP>(args, stream) : launch_direct_one<kDM, NW, WM, false, false, false, NP>(args, stream);
 }
 
 }  // namespace dmoe

@@ -8,7 +8,7 @@ int launch_direct_bf16_small(const GmmArgs &args, int tile_rows, bool trans_b, b
 int launch_direct_bf16_256(const GmmArgs &args, bool trans_b, bool swiglu, hipStream_t stream);
 
 // Preconditions (checked by the caller): bf16, K % 32 == 0, N % 8 == 0, K * N * 2 < 2^32.
-// tile_rows: 256 (8 wavefronts, alternating phases), 128 (4 wavefronts) or 64 (4 computing + 2 copying wavefronts).
+// tile_rows: 256 (gmm_tile256.h), 128 (4 wavefronts) or 64 (4 computing + 2 copying wavefronts) (gmm_direct.h).
 int launch_direct_bf16(const GmmArgs &args, int tile_rows, bool trans_b, bool swiglu, hipStream_t stream) {
     if (tile_rows == 64 || tile_rows == 128) return launch_direct_bf16_small(args, tile_rows, trans_b, swiglu, stream);
     return launch_direct_bf16_256(args, trans_b, swiglu, stream);

@@ -32,12 +32,14 @@ MEASURED_TRAFFIC = {"C2": 6.11e9, "C4": 1.551e9, "C5": 13.95e9}
 def _tile_rows(w) -> int:
     """Tile rows the gate-up launch gets: mirrors launch_by_rows (csrc/gmm.hip)."""
     import torch
-    avg = w.R // w.E
-    tile = 64 if avg <= 64 else (128 if avg <= 160 else 256)
     cus = torch.cuda.get_device_properties(0).multi_processor_count
     n_tiles = (w.I + 127) // 128
-    while tile > 64 and (w.R // tile + (w.E + 1) // 2) * n_tiles * 2 < cus:
-        tile //= 2
+    tile = 256
+    if w.fp8 or (w.R // 256 + (w.E + 1) // 2) * n_tiles < cus:
+        avg = w.R // w.E
+        tile = 64 if avg <= 64 else (128 if avg <= 160 else 256)
+        while tile > 64 and (w.R // tile + (w.E + 1) // 2) * n_tiles * 2 < cus:
+            tile //= 2
     return tile
 
 
@@ -224,7 +226,8 @@ def main() -> int:
         peak = PEAK_BF16_TFLOPS
         tile = _tile_rows(w)
         direct = w.d % 32 == 0
-        kernel = (f"dmoe::gmm_direct_kernel<{tile}, .., [K,N] weights, swiglu, bf16>" if direct
+        kernel = (("dmoe::gmm_tile256_kernel<[K,N] weights, swiglu>" if tile == 256 else
+                   f"dmoe::gmm_direct_kernel<{tile}, .., [K,N] weights, swiglu, bf16>") if direct
                   else f"dmoe::gmm_kernel<{tile}, 256, .., swiglu, bf16>") + " (gate-up projection with fused SiLU*mul)"
     up_flops = 2.0 * w.R * w.d * 2 * w.I
     down_flops = 2.0 * w.R * w.I * w.d

@@ -466,7 +466,7 @@ static int bind_state(GmmArgs &args, void *state, void *workspace, size_t worksp
 
 template <bool TRANS_B, bool SWIGLU, bool FP8>
 static int launch_by_rows(const GmmArgs &args, hipStream_t stream) {
-    // rows per expert on average decide the m-tile; the host does not know the split
+    // the host does not know how the rows split over the experts
     const long long avg = args.rows / (args.E > 0 ? args.E : 1);
     switch (g_variant) {
         case 1: return launch_one<256, 256, 2, 2, TRANS_B, SWIGLU, FP8>(args, stream);
@@ -475,10 +475,17 @@ static int launch_by_rows(const GmmArgs &args, hipStream_t stream) {
         case 4: return launch_one<256, 256, 2, 4, TRANS_B, SWIGLU, FP8>(args, stream);
         default: break;
     }
-    int tile_rows = avg <= 64 ? 64 : (avg <= 160 ? 128 : 256);
-    // a tile size that would leave more than half of the CUs without a tile is halved (small problems: latency counts)
+    // Tile rows.  Every m-tile streams its 256 columns of the weights through the CU whatever its rows, so fewer, taller
+    // tiles move fewer bytes (decode-sized batches: 8 tiles of 256 rows instead of 12 of 64 on the Zipf batch, 10 % off the
+    // gate-up launch) and a tile's empty row fragments cost no MFMAs: 256 rows wherever such tiles fill the CUs.  Else
+    // the rows per expert on average decide, and a size that would leave more than half of the CUs without a tile is
+    // halved (small problems: latency counts).
     const long long n_tiles = ((SWIGLU ? args.N / 2 : args.N) + (SWIGLU ? 127 : 255)) / (SWIGLU ? 128 : 256);
-    while (tile_rows > 64 && (args.rows / tile_rows + (args.E + 1) / 2) * n_tiles * 2 < device_cus()) tile_rows /= 2;
+    int tile_rows = 256;
+    if (FP8 || (args.rows / 256 + (args.E + 1) / 2) * n_tiles < device_cus()) {
+        tile_rows = avg <= 64 ? 64 : (avg <= 160 ? 128 : 256);
+        while (tile_rows > 64 && (args.rows / tile_rows + (args.E + 1) / 2) * n_tiles * 2 < device_cus()) tile_rows /= 2;
+    }
     if (g_variant >= 5) tile_rows = g_variant == 5 ? 64 : (g_variant == 6 ? 128 : 256);   // direct kernel, fixed tile rows
     if constexpr (!FP8) {
         // global -> LDS direct path: whole stages of 32 k, 32-bit offsets inside one expert's weights

@@ -32,6 +32,9 @@ SIGNATURES = {
     "dmoe_move_row_infos": (c_int, [c_void_p, c_int, c_void_p, c_int64, c_void_p]),
     "dmoe_expert_batch_sizes": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_int, c_void_p]),
     "dmoe_host_mappings": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_void_p]),
+    "dmoe_metadata_wire_bytes": (c_int, [c_void_p, POINTER(c_size_t)]),
+    "dmoe_metadata_serialize": (c_int, [c_void_p, c_void_p, c_size_t]),
+    "dmoe_metadata_parse": (c_int, [c_void_p, c_size_t, c_void_p]),
     "dmoe_permute": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int, c_void_p,
                              c_void_p]),
     "dmoe_gather_rows": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int, c_void_p]),
@@ -57,6 +60,29 @@ TEST_HOOKS = {
     "dmoe_gmm_tune": (c_int, [c_int]),
 }
 GMM_STATE_BYTES = 33024
+
+
+
+class MetadataView(ctypes.Structure):
+    """dmoe_metadata_view of include/dmoe.h."""
+    _fields_ = [("shape", c_void_p), ("n_shape", ctypes.c_uint64), ("dtype", c_void_p), ("n_dtype", ctypes.c_uint64),
+                ("layer_id", ctypes.c_int32),
+                ("req_ids", c_void_p), ("n_req_ids", ctypes.c_uint64), ("exp_ids", c_void_p), ("n_exp_ids", ctypes.c_uint64),
+                ("attn_dp_ranks", c_void_p), ("n_attn_dp_ranks", ctypes.c_uint64),
+                ("init_prefill_lens", c_void_p), ("n_init_prefill_lens", ctypes.c_uint64),
+                ("topk_weights", c_void_p), ("n_topk_weights", ctypes.c_uint64)]
+
+
+class MetadataLayout(ctypes.Structure):
+    """dmoe_metadata_layout of include/dmoe.h."""
+    _fields_ = [("off_shape", ctypes.c_uint64), ("n_shape", ctypes.c_uint64), ("off_dtype", ctypes.c_uint64),
+                ("n_dtype", ctypes.c_uint64), ("layer_id", ctypes.c_int32),
+                ("off_req_ids", ctypes.c_uint64), ("n_req_ids", ctypes.c_uint64),
+                ("off_exp_ids", ctypes.c_uint64), ("n_exp_ids", ctypes.c_uint64),
+                ("off_attn_dp_ranks", ctypes.c_uint64), ("n_attn_dp_ranks", ctypes.c_uint64),
+                ("off_init_prefill_lens", ctypes.c_uint64), ("n_init_prefill_lens", ctypes.c_uint64),
+                ("off_topk_weights", ctypes.c_uint64), ("n_topk_weights", ctypes.c_uint64)]
+
 
 _lib = None
 

@@ -80,3 +80,89 @@ extern "C" int dmoe_host_mappings(const int32_t *exp_ids, int64_t n, int n_exper
     for (int64_t i = 0; i < n; ++i) mappings[i] = --cursor[(size_t)exp_ids[i]];
     return DMOE_OK;
 }
+
+// ---- wire format of a batch's bookkeeping -------------------------------------------------------------
+// The reference sends Metadata between its workers as a cereal BinaryOutputArchive of the fields in the order of
+// Metadata::serialize (csrc/include/datatypes.hpp:223-226; csrc/include/utils.hpp:150-174).  cereal (v1.3, a header
+// library the reference builds against, not part of its tree) writes, in the byte order of the host: an arithmetic
+// value as its bytes; a std::vector of arithmetic values and a std::string as the element count (cereal::size_type,
+// 64 bits) followed by the elements' bytes; a struct with a serialize member as its fields one after the other.
+// So a blob is   u64 n, u64 shape[n] | u64 n, char dtype[n] | i32 layer_id | u64 n, i32 req_ids[n] | u64 n, i32
+// exp_ids[n] | u64 n, i32 attn_dp_ranks[n] | u64 n, i32 init_prefill_lens[n] | u64 n, f32 topk_weights[n].
+
+namespace {
+
+struct Field { const void *data; uint64_t count; size_t elem; };
+
+void fields_of(const dmoe_metadata_view &m, Field (&f)[7]) {
+    f[0] = {m.shape, m.n_shape, 8};
+    f[1] = {m.dtype, m.n_dtype, 1};
+    f[2] = {m.req_ids, m.n_req_ids, 4};
+    f[3] = {m.exp_ids, m.n_exp_ids, 4};
+    f[4] = {m.attn_dp_ranks, m.n_attn_dp_ranks, 4};
+    f[5] = {m.init_prefill_lens, m.n_init_prefill_lens, 4};
+    f[6] = {m.topk_weights, m.n_topk_weights, 4};
+}
+
+}  // namespace
+
+extern "C" int dmoe_metadata_wire_bytes(const dmoe_metadata_view *m, size_t *bytes) {
+    DMOE_REQUIRE(m && bytes, DMOE_ERR_ARG, "dmoe_metadata_wire_bytes: null pointer");
+    Field f[7];
+    fields_of(*m, f);
+    size_t total = 4;   // layer_id
+    for (const Field &x : f) {
+        DMOE_REQUIRE(x.count < (1ull << 40), DMOE_ERR_SHAPE, "dmoe_metadata_wire_bytes: a list of %llu entries", (unsigned long long)x.count);
+        DMOE_REQUIRE(x.count == 0 || x.data, DMOE_ERR_ARG, "dmoe_metadata_wire_bytes: null list with %llu entries", (unsigned long long)x.count);
+        total += 8 + (size_t)x.count * x.elem;
+    }
+    *bytes = total;
+    return DMOE_OK;
+}
+
+extern "C" int dmoe_metadata_serialize(const dmoe_metadata_view *m, void *out, size_t out_bytes) {
+    size_t need = 0;
+    int rc = dmoe_metadata_wire_bytes(m, &need);
+    if (rc != DMOE_OK) return rc;
+    DMOE_REQUIRE(out && out_bytes >= need, DMOE_ERR_WORKSPACE, "dmoe_metadata_serialize: %zu bytes needed, %zu given", need, out_bytes);
+    Field f[7];
+    fields_of(*m, f);
+    char *p = (char *)out;
+    auto put_list = [&](const Field &x) {
+        std::memcpy(p, &x.count, 8); p += 8;
+        if (x.count) std::memcpy(p, x.data, (size_t)x.count * x.elem);
+        p += (size_t)x.count * x.elem;
+    };
+    put_list(f[0]);
+    put_list(f[1]);
+    std::memcpy(p, &m->layer_id, 4); p += 4;
+    for (int i = 2; i < 7; ++i) put_list(f[i]);
+    return DMOE_OK;
+}
+
+extern "C" int dmoe_metadata_parse(const void *blob, size_t blob_bytes, dmoe_metadata_layout *out) {
+    DMOE_REQUIRE(blob && out, DMOE_ERR_ARG, "dmoe_metadata_parse: null pointer");
+    const char *base = (const char *)blob;
+    size_t pos = 0;
+    bool ok = true;
+    auto take_list = [&](size_t elem, uint64_t *offset, uint64_t *count) {
+        if (!ok || blob_bytes - pos < 8) { ok = false; return; }
+        uint64_t n;
+        std::memcpy(&n, base + pos, 8);
+        pos += 8;
+        if (n > (blob_bytes - pos) / elem) { ok = false; return; }
+        *offset = pos; *count = n;
+        pos += (size_t)n * elem;
+    };
+    take_list(8, &out->off_shape, &out->n_shape);
+    take_list(1, &out->off_dtype, &out->n_dtype);
+    if (ok && blob_bytes - pos >= 4) { std::memcpy(&out->layer_id, base + pos, 4); pos += 4; } else ok = false;
+    take_list(4, &out->off_req_ids, &out->n_req_ids);
+    take_list(4, &out->off_exp_ids, &out->n_exp_ids);
+    take_list(4, &out->off_attn_dp_ranks, &out->n_attn_dp_ranks);
+    take_list(4, &out->off_init_prefill_lens, &out->n_init_prefill_lens);
+    take_list(4, &out->off_topk_weights, &out->n_topk_weights);
+    DMOE_REQUIRE(ok, DMOE_ERR_SHAPE, "dmoe_metadata_parse: the blob of %zu bytes ends inside a field (at byte %zu)", blob_bytes, pos);
+    DMOE_REQUIRE(pos == blob_bytes, DMOE_ERR_SHAPE, "dmoe_metadata_parse: %zu bytes behind the last field", blob_bytes - pos);
+    return DMOE_OK;
+}

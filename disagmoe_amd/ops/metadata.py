@@ -3,8 +3,8 @@
 Mirror of the part of the reference's ``Metadata`` (csrc/include/datatypes.hpp:135-501) that the
 expert step reads and writes (disagmoe/frontend/engine.py:683-739): the lists live on the host as
 they do there, the sorting and moving runs in the C++ library (no Python loops over rows), and what
-reaches the device is a row mapping for ``permute_tokens``.  The wire format (cereal field order,
-datatypes.hpp:223-226) belongs to the transport and is not part of this package.
+reaches the device is a row mapping for ``permute_tokens``.  ``serialize`` / ``deserialize`` read and
+write the bytes the reference's workers exchange for a batch (cereal field order, datatypes.hpp:223-226).
 """
 from __future__ import annotations
 
@@ -143,6 +143,41 @@ class Metadata:
         if topk == 1:
             return
         self.shape = [self.shape[0] // topk] + list(self.shape[1:])
+
+    def serialize(self) -> bytes:
+        """The bytes the reference's workers exchange for this Metadata: cereal's binary archive of the fields in the
+        order of ``Metadata::serialize`` (datatypes.hpp:223-226; ``cerealize``, utils.hpp:150-157)."""
+        import ctypes
+        keep = [np.ascontiguousarray(np.asarray(self.shape, dtype=np.uint64)), np.frombuffer(self.dtype.encode(), dtype=np.uint8),
+                _i32(self.req_ids), _i32(self.exp_ids), _i32(self.attn_dp_ranks), _i32(self.init_prefill_lens),
+                np.ascontiguousarray(np.asarray(self.topk_weights, dtype=np.float32))]
+        p = [a.ctypes.data if a.size else None for a in keep]
+        view = _lib.MetadataView(p[0], keep[0].size, p[1], keep[1].size, int(self.layer_id), p[2], keep[2].size, p[3],
+                                 keep[3].size, p[4], keep[4].size, p[5], keep[5].size, p[6], keep[6].size)
+        need = ctypes.c_size_t(0)
+        _lib.call("dmoe_metadata_wire_bytes", ctypes.byref(view), ctypes.byref(need))
+        out = ctypes.create_string_buffer(need.value)
+        _lib.call("dmoe_metadata_serialize", ctypes.byref(view), out, need.value)
+        return out.raw
+
+    @staticmethod
+    def deserialize(blob: bytes) -> "Metadata":
+        """Inverse of :meth:`serialize` (``decerealize``, utils.hpp:167-174).  Raises ``DmoeError`` on a blob that ends
+        early or has bytes left over."""
+        import ctypes
+        lay = _lib.MetadataLayout()
+        buf = (ctypes.c_char * len(blob)).from_buffer_copy(blob)
+        _lib.call("dmoe_metadata_parse", buf, len(blob), ctypes.byref(lay))
+
+        def take(off, n, dtype):
+            return np.frombuffer(blob, dtype=dtype, count=int(n), offset=int(off)).tolist()
+
+        return Metadata(shape=take(lay.off_shape, lay.n_shape, "<u8"),
+                        dtype=bytes(blob[lay.off_dtype:lay.off_dtype + lay.n_dtype]).decode(), layer_id=int(lay.layer_id),
+                        req_ids=take(lay.off_req_ids, lay.n_req_ids, "<i4"), exp_ids=take(lay.off_exp_ids, lay.n_exp_ids, "<i4"),
+                        attn_dp_ranks=take(lay.off_attn_dp_ranks, lay.n_attn_dp_ranks, "<i4"),
+                        init_prefill_lens=take(lay.off_init_prefill_lens, lay.n_init_prefill_lens, "<i4"),
+                        topk_weights=take(lay.off_topk_weights, lay.n_topk_weights, "<f4"))
 
     @staticmethod
     def merge_by_exp_ids(metas: Sequence["Metadata"], n_expert: Optional[int] = None):

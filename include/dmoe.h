@@ -139,6 +139,38 @@ int dmoe_expert_batch_sizes(const int32_t *exp_ids, int64_t n, int n_expert, con
  * holds 32).  dmoe_route is the device form of the same rule. */
 int dmoe_host_mappings(const int32_t *exp_ids, int64_t n, int n_expert, int64_t *mappings, int64_t *exp_cnt);
 
+/* Wire format of a batch's bookkeeping: the bytes the reference's workers exchange for a Metadata, a cereal
+ * BinaryOutputArchive of its fields in the order of Metadata::serialize (csrc/include/datatypes.hpp:223-226, written
+ * and read by cerealize / decerealize, csrc/include/utils.hpp:150-174), host byte order:
+ *     u64 n, u64 shape[n] | u64 n, char dtype[n] | i32 layer_id | u64 n, i32 req_ids[n] | u64 n, i32 exp_ids[n] |
+ *     u64 n, i32 attn_dp_ranks[n] | u64 n, i32 init_prefill_lens[n] | u64 n, f32 topk_weights[n]
+ * dmoe_metadata_serialize writes the lists of a view (host pointers) into `out` (dmoe_metadata_wire_bytes bytes);
+ * dmoe_metadata_parse checks a blob and reports where each list lies in it (byte offsets: the lists of a blob are
+ * not aligned) and how many entries it has.  A blob that ends early or has bytes left over is DMOE_ERR_SHAPE. */
+typedef struct dmoe_metadata_view {
+    const uint64_t *shape; uint64_t n_shape;
+    const char *dtype; uint64_t n_dtype;
+    int32_t layer_id;
+    const int32_t *req_ids; uint64_t n_req_ids;
+    const int32_t *exp_ids; uint64_t n_exp_ids;
+    const int32_t *attn_dp_ranks; uint64_t n_attn_dp_ranks;
+    const int32_t *init_prefill_lens; uint64_t n_init_prefill_lens;
+    const float *topk_weights; uint64_t n_topk_weights;
+} dmoe_metadata_view;
+typedef struct dmoe_metadata_layout {
+    uint64_t off_shape, n_shape;
+    uint64_t off_dtype, n_dtype;
+    int32_t layer_id;
+    uint64_t off_req_ids, n_req_ids;
+    uint64_t off_exp_ids, n_exp_ids;
+    uint64_t off_attn_dp_ranks, n_attn_dp_ranks;
+    uint64_t off_init_prefill_lens, n_init_prefill_lens;
+    uint64_t off_topk_weights, n_topk_weights;
+} dmoe_metadata_layout;
+int dmoe_metadata_wire_bytes(const dmoe_metadata_view *m, size_t *bytes);
+int dmoe_metadata_serialize(const dmoe_metadata_view *m, void *out, size_t out_bytes);
+int dmoe_metadata_parse(const void *blob, size_t blob_bytes, dmoe_metadata_layout *out);
+
 /* ---- row movement -------------------------------------------------------
  * dmoe_permute replaces permute_tokens_cuda(tokens, mappings, stream)
  * (csrc/include/permute.h:8, csrc/cuda_ops/permute.cu:86-112, bound at

@@ -63,3 +63,43 @@ def test_graph_replays_equal_eager(name, T, fp8):
         eager = _step(layer, xr.to(dev()), lr.to(dev()), w.k)   # eager work between replays, different routing
         torch.cuda.synchronize()
         assert torch.equal(got, eager), f"replay {rep} differs from the eager step"
+
+
+def test_expert_worker_step_recorded_once():
+    # the device half of process_batch_expert (uploads from pinned staging into the static buffers, FFN, scale + return
+    # permute) recorded once; every replay follows the host half of a new batch of the same size
+    from disagmoe_amd.config import ModelConfig
+    from disagmoe_amd.executor import ExpertsExecutor
+    from disagmoe_amd.expert_layer import ExpertWorker
+    from test_gpu_layer import _expert_step_case, _expert_step_reference
+    announce(test="graph_expert_worker")
+    E, d, I, top_k, R = 8, 512, 768, 2, 192
+    cfg = ModelConfig(hidden_size=d, num_layers=1, num_heads=8, num_kv_heads=8, num_experts=E, intermediate_size=I,
+                      layer_ids=[0], top_k=top_k, max_batch_size_expert=256)
+    ex = ExpertsExecutor(cfg, init_std=0.02)
+    worker = ExpertWorker(ex, top_k=top_k)
+    x_static = torch.zeros(R, d, dtype=torch.bfloat16, device=dev())
+    meta, x, *case = _expert_step_case(E, d, R, top_k, seed=100)
+    x_static.copy_(x)
+    side = torch.cuda.Stream(device=dev())
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        worker.process_batch_expert(meta, x_static)                    # warm-up outside the recording
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    meta, x, *case = _expert_step_case(E, d, R, top_k, seed=101)
+    x_static.copy_(x)
+    worker.stage(meta)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out_static = worker.run(0, x_static)
+    for rep in range(4):
+        meta, x, *case = _expert_step_case(E, d, R, top_k, seed=200 + rep)
+        x_static.copy_(x)
+        worker.stage(meta)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out_static.clone()
+        ref = _expert_step_reference(ex.operators[0], x, *case, E, False)      # eager work between the replays
+        torch.cuda.synchronize()
+        assert torch.equal(got, ref), f"replay {rep}"

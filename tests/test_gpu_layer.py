@@ -137,3 +137,62 @@ def test_process_batch_expert(top_k):
     moved = torch.empty_like(y_dev)
     moved[torch.tensor(mapping, device=dev())] = y_dev
     assert torch.equal(out, moved)
+
+
+def _expert_step_case(E, d, R, top_k, seed):
+    from disagmoe_amd.ops.metadata import Metadata
+    g = torch.Generator().manual_seed(seed)
+    exp_ids = torch.sort(torch.randint(0, E, (R,), generator=g)).values.tolist()
+    req_ids = torch.randperm(R, generator=g).tolist()
+    lens = torch.where(torch.rand(R, generator=g) < 0.5, -1, 8).tolist()
+    dp = torch.randint(0, 2, (R,), generator=g).tolist()
+    weights = torch.rand(R, generator=g).tolist() if top_k > 1 else []
+    x = torch.randn(R, d, generator=g).to(torch.bfloat16)
+    meta = Metadata(shape=[R, d], layer_id=0, req_ids=list(req_ids), exp_ids=list(exp_ids), attn_dp_ranks=list(dp),
+                    init_prefill_lens=list(lens), topk_weights=list(weights))
+    return meta, x, exp_ids, req_ids, lens, dp, weights
+
+
+def _expert_step_reference(op, x, exp_ids, req_ids, lens, dp, weights, E, pairing):
+    """Statement by statement what engine.py:705-734 computes, with torch on the device: the FFN of the layer under
+    test, the scale, the scatter to the return order."""
+    sizes = routing.expert_batch_sizes(exp_ids, E).tolist()
+    y = op.forward(len(exp_ids), x.to(dev()), torch.tensor(sizes, device=dev()))
+    mapping = routing.sort_by_prefill_order(req_ids, dp, lens)
+    if weights:
+        w = list(weights)
+        if pairing:   # the lists were reordered before the weights were read: position r holds the weight of the row that moves there
+            w = routing.apply_row_mapping(weights, mapping)
+        y = y * torch.tensor(w, dtype=torch.bfloat16, device=dev()).view(-1, 1)
+    moved = torch.empty_like(y)
+    moved[torch.tensor(mapping, device=dev())] = y
+    return moved
+
+
+@pytest.mark.parametrize("pairing", [False, True])
+def test_expert_worker_static_buffers(pairing):
+    # consecutive steps of different sizes through one worker's static buffers, one of them larger than the buffers;
+    # with the reference's weight pairing and with each row's own weight
+    from disagmoe_amd.config import ModelConfig
+    from disagmoe_amd.executor import ExpertsExecutor
+    from disagmoe_amd.expert_layer import ExpertWorker
+    announce(test="expert_worker", pairing=pairing)
+    E, d, I, top_k = 4, 512, 768, 2
+    cfg = ModelConfig(hidden_size=d, num_layers=1, num_heads=8, num_kv_heads=8, num_experts=E, intermediate_size=I,
+                      layer_ids=[0], top_k=top_k, max_batch_size_expert=256)
+    ex = ExpertsExecutor(cfg, init_std=0.02)
+    worker = ExpertWorker(ex, top_k=top_k, reference_weight_pairing=pairing)
+    buffers = (worker.static_mappings.data_ptr(), worker.static_batch_sizes.data_ptr(), worker.static_weights.data_ptr())
+    for seed, R in [(1, 200), (2, 256), (3, 90), (4, 300), (5, 120)]:          # 300 rows: beyond max_batch_size_expert
+        meta, x, exp_ids, req_ids, lens, dp, weights = _expert_step_case(E, d, R, top_k, seed)
+        out, new_meta = worker.process_batch_expert(meta, x.to(dev()))
+        ref = _expert_step_reference(ex.operators[0], x, exp_ids, req_ids, lens, dp, weights, E, pairing)
+        assert torch.equal(out, ref), (seed, R)
+        assert new_meta.layer_id == 1 and new_meta.exp_ids == []
+    assert buffers == (worker.static_mappings.data_ptr(), worker.static_batch_sizes.data_ptr(),
+                       worker.static_weights.data_ptr())
+    if not pairing:      # the two pairings differ whenever the return mapping moves rows
+        meta, x, exp_ids, req_ids, lens, dp, weights = _expert_step_case(E, d, 100, top_k, 9)
+        other = _expert_step_reference(ex.operators[0], x, exp_ids, req_ids, lens, dp, weights, E, True)
+        out, _ = worker.process_batch_expert(meta, x.to(dev()))
+        assert not torch.equal(out, other)

@@ -147,3 +147,43 @@ def test_merge_by_exp_ids_matches_oracle():
     weights = cat("topk_weights") + [0.0] * 9      # the last batch came without weights
     assert merged.topk_weights == routing.apply_row_mapping(weights, mappings)
     assert merged.get_expert_batch_sizes(E) == cnt_ref
+
+
+def test_wire_format_golden_blobs(golden_dir):
+    # byte-exact writer and reader against hand-assembled blobs (cereal binary archive, field order of
+    # Metadata::serialize, datatypes.hpp:223-226)
+    import json
+    import os
+    from disagmoe_amd.ops.metadata import Metadata
+    from disagmoe_amd._lib import DmoeError
+    for case in json.load(open(os.path.join(golden_dir, "metadata_wire.json"))):
+        blob = bytes.fromhex(case["hex"].replace(" ", ""))
+        meta = Metadata(**case["fields"])
+        assert meta.serialize() == blob
+        back = Metadata.deserialize(blob)
+        for name, value in case["fields"].items():
+            assert getattr(back, name) == value, name
+        assert back.serialize() == blob
+        # a blob cut short or with bytes left over is refused
+        for bad in (blob[:-1], blob + b"\0", blob[:13]):
+            with pytest.raises(DmoeError):
+                Metadata.deserialize(bad)
+    # a count that points past the end of the blob
+    with pytest.raises(DmoeError):
+        Metadata.deserialize((2 ** 40).to_bytes(8, "little") + b"\0" * 64)
+
+
+def test_wire_format_round_trip_after_the_expert_step():
+    from disagmoe_amd.ops.metadata import Metadata
+    rng = np.random.default_rng(3)
+    n = 257
+    meta = Metadata(shape=[n, 4096], layer_id=7, req_ids=rng.integers(0, 10 ** 6, n).tolist(),
+                    exp_ids=rng.integers(0, 64, n).tolist(), attn_dp_ranks=rng.integers(0, 4, n).tolist(),
+                    init_prefill_lens=rng.choice([-1, 5, 900], n).tolist(), topk_weights=rng.random(n, dtype=np.float32).tolist())
+    blob = meta.serialize()
+    assert len(blob) == 8 * 3 + (8 + 4) + 4 + 5 * 8 + 5 * 4 * n
+    back = Metadata.deserialize(blob)
+    assert back == meta
+    back.sort_by_prefill_order()
+    again = Metadata.deserialize(back.serialize())
+    assert again == back and again.exp_ids == []

@@ -24,9 +24,13 @@ PEAK_HBM_GBS = 8000.0
 PEAK_BF16_TFLOPS = 2500.0
 PEAK_FP8_TFLOPS = 5000.0
 
-# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc runs (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0,
-# the factors read off a 1 GiB copy in the same runs: profiles/expert_layer_c2_hbm_traffic.md); None = not measured.
-MEASURED_TRAFFIC = {"C2": 6.11e9, "C4": 1.551e9, "C5": 13.95e9}
+# Bytes per launch of the dominant kernel that crossed the L2 boundary, from rocprofv3 --pmc runs of this script
+# (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, the factors read off a 1 GiB copy in the same runs).  A bench run does not
+# measure them: they are read off the committed summaries named here.  None = not measured.
+MEASURED_TRAFFIC = {"C2": (7.654e9, "profiles/expert_layer_c2_hbm_traffic.md"),
+                    "C3": (1.927e9, "profiles/expert_layer_c5_c4_c3_hbm_traffic.md"),
+                    "C4": (2.152e9, "profiles/expert_layer_c5_c4_c3_hbm_traffic.md"),
+                    "C5": (13.357e9, "profiles/expert_layer_c5_c4_c3_hbm_traffic.md")}
 
 
 def _tile_rows(w) -> int:
@@ -107,6 +111,8 @@ def main() -> int:
     ap.add_argument("--variant", type=int, default=0, help="grouped GEMM tile variant (tuning)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--kernel-iters", type=int, default=10)
+    ap.add_argument("--no-split", action="store_true",
+                    help="grouped GEMMs without a workspace: the tiles of the last round are not cut along K (comparison)")
     ap.add_argument("--copy-probe-mib", type=int, default=0,
                     help="also run a plain device copy of this many MiB (scales the FETCH_SIZE/WRITE_SIZE counters)")
     args = ap.parse_args()
@@ -143,6 +149,12 @@ def main() -> int:
         layer.w2_weight = torch.nn.Parameter(w2, requires_grad=False)
         layer.enable_cache = False
         layer.gmm_cache_max_batch_size = 0
+    # state block and workspace of the layer's launches, as MoEExperts.create_weights sets them up
+    ws_size, args_ptr = gg.get_arguments(w.E, dev)
+    gemm_state = dict(arguments_ptr=args_ptr,
+                      workspace=None if args.no_split else torch.empty([ws_size], dtype=torch.uint8, device=dev))
+    if not w.fp8:
+        layer.arguments_ptr, layer.workspace = gemm_state["arguments_ptr"], gemm_state["workspace"]
     torch.cuda.synchronize()
 
     def step():
@@ -188,6 +200,14 @@ def main() -> int:
 
     ms, _ = _event_ms(lambda: memory.route_tokens(ids, w.E), it, plug=plug)
     stages["route"] = {"ms": ms, "GB/s": w.route_bytes / ms / 1e6}
+    def gemm_ms(fn):
+        """(ms per launch with 5 launches inside one event pair: what a profiler's kernel duration compares with; ms of
+        one launch inside its own event pair, which holds the events' own packets as well)"""
+        def many():
+            for _ in range(5):
+                fn()
+        return _event_ms(many, max(2, it // 2))[0] / 5, _event_ms(fn, it)[0]
+
     def sustained_ms(fn, n=10):
         """ms per launch when n launches follow each other inside one event interval: a launch's ramp-up overlaps the
         drain of the one before it, as it does behind another kernel in a running step"""
@@ -207,8 +227,9 @@ def main() -> int:
         xq, xs = gg.quantize_rows(permuted)
         h = gg.gmm_fp8_swiglu(xq, xs, layer.w13_q, layer.w13_scale, batch_sizes)
         hq, hs = gg.quantize_rows(h)
-        up_ms, _ = _event_ms(lambda: gg.gmm_fp8_swiglu(xq, xs, layer.w13_q, layer.w13_scale, batch_sizes, c=h), it)
-        down_ms, _ = _event_ms(lambda: gg.gmm_fp8(hq, hs, layer.w2_q, layer.w2_scale, batch_sizes), it)
+        up_ms, up_single = gemm_ms(lambda: gg.gmm_fp8_swiglu(xq, xs, layer.w13_q, layer.w13_scale, batch_sizes, c=h))
+        y_buf = torch.empty((w.R, w.d), dtype=torch.bfloat16, device=dev)
+        down_ms, down_single = gemm_ms(lambda: gg.gmm_fp8(hq, hs, layer.w2_q, layer.w2_scale, batch_sizes, c=y_buf))
         q_ms, _ = _event_ms(lambda: gg.quantize_rows(h), it)
         stages["quant_rows"] = {"ms": q_ms, "GB/s": 3.0 * w.R * w.I / q_ms / 1e6}       # the [R, I] intermediate
         pq_ms, _ = _event_ms(lambda: memory.permute_quantize(x, mappings), it)
@@ -219,10 +240,10 @@ def main() -> int:
         kernel = (f"dmoe::gmm_kernel<{tile}, 256, .., swiglu, fp8>" if w.d % 64
                   else f"dmoe::gmm_direct_kernel<{tile}, .., swiglu, fp8>") + " (gate-up projection with fused SiLU*mul)"
     else:
-        h = gg.gmm_swiglu(permuted, layer.w13_weight, batch_sizes)
-        up_ms, _ = _event_ms(lambda: gg.gmm_swiglu(permuted, layer.w13_weight, batch_sizes, c=h), it)
+        h = gg.gmm_swiglu(permuted, layer.w13_weight, batch_sizes, **gemm_state)
+        up_ms, up_single = gemm_ms(lambda: gg.gmm_swiglu(permuted, layer.w13_weight, batch_sizes, c=h, **gemm_state))
         y_buf = torch.empty((w.R, w.d), dtype=torch.bfloat16, device=dev)
-        down_ms, _ = _event_ms(lambda: gg.gmm(h, layer.w2_weight, batch_sizes, c=y_buf), it)
+        down_ms, down_single = gemm_ms(lambda: gg.gmm(h, layer.w2_weight, batch_sizes, c=y_buf, **gemm_state))
         peak = PEAK_BF16_TFLOPS
         tile = _tile_rows(w)
         direct = w.d % 32 == 0
@@ -231,8 +252,17 @@ def main() -> int:
                   else f"dmoe::gmm_kernel<{tile}, 256, .., swiglu, bf16>") + " (gate-up projection with fused SiLU*mul)"
     up_flops = 2.0 * w.R * w.d * 2 * w.I
     down_flops = 2.0 * w.R * w.I * w.d
-    stages["gemm_gate_up"] = {"ms": up_ms, "TFLOP/s": up_flops / up_ms / 1e9, "frac_mfma": up_flops / up_ms / 1e9 / peak}
-    stages["gemm_down"] = {"ms": down_ms, "TFLOP/s": down_flops / down_ms / 1e9, "frac_mfma": down_flops / down_ms / 1e9 / peak}
+    if not w.fp8:
+        # yardstick, not part of the path: the vendor library's dense GEMM of the gate-up launch's flop count
+        # ([R, d] x [d, 2I], one expert's weights, no SiLU*mul), timed the same way on the same box
+        dense_c = torch.empty((w.R, 2 * w.I), dtype=torch.bfloat16, device=dev)
+        lib_ms, _ = gemm_ms(lambda: torch.mm(permuted, layer.w13_weight[0], out=dense_c))
+        stages["library_dense_gemm"] = {"ms": lib_ms, "TFLOP/s": up_flops / lib_ms / 1e9, "frac_mfma": up_flops / lib_ms / 1e9 / peak,
+                                        "what": "torch.mm (hipBLASLt) on [R, d] x [d, 2I]: the flop count of the gate-up launch as "
+                                                "one dense GEMM without the epilogue; a yardstick for what this chip sustains"}
+        del dense_c
+    stages["gemm_gate_up"] = {"ms": up_ms, "ms_single_launch": up_single, "TFLOP/s": up_flops / up_ms / 1e9, "frac_mfma": up_flops / up_ms / 1e9 / peak}
+    stages["gemm_down"] = {"ms": down_ms, "ms_single_launch": down_single, "TFLOP/s": down_flops / down_ms / 1e9, "frac_mfma": down_flops / down_ms / 1e9 / peak}
     stages["gemm_total"] = {"ms": up_ms + down_ms, "TFLOP/s": w.gemm_flops / (up_ms + down_ms) / 1e9,
                             "frac_mfma": w.gemm_flops / (up_ms + down_ms) / 1e9 / peak}
     y = layer.forward(w.R, permuted, batch_sizes)
@@ -250,15 +280,18 @@ def main() -> int:
     stages["gemm_down"].update({"GB/s": down_bytes / down_ms / 1e6, "frac_hbm": down_bytes / down_ms / 1e6 / PEAK_HBM_GBS})
 
     achieved = up_flops / up_ms / 1e9
+    traffic, traffic_source = MEASURED_TRAFFIC.get(args.config, (None, None))
+    if args.no_split:
+        traffic, traffic_source = None, None
     if up_flops / up_bytes < peak * 1e12 / (PEAK_HBM_GBS * 1e9):
         # fewer flops per byte than the ridge of the roofline (decode-sized batches): streaming the weights bounds it
         roofline = {"kernel": kernel, "bound": "hbm", "achieved": up_bytes / up_ms / 1e6, "peak": PEAK_HBM_GBS,
                     "unit": "GB/s", "frac": up_bytes / up_ms / 1e6 / PEAK_HBM_GBS,
-                    "traffic": MEASURED_TRAFFIC.get(args.config), "bytes_per_launch": up_bytes,
+                    "traffic": traffic, "traffic_source": traffic_source, "bytes_per_launch": up_bytes,
                     "flops_per_launch": up_flops, "avg_launch_ms": up_ms}
     else:
         roofline = {"kernel": kernel, "bound": "mfma", "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
-                    "frac": achieved / peak, "traffic": MEASURED_TRAFFIC.get(args.config),
+                    "frac": achieved / peak, "traffic": traffic, "traffic_source": traffic_source,
                     "flops_per_launch": up_flops, "avg_launch_ms": up_ms}
 
     record = {
@@ -267,8 +300,13 @@ def main() -> int:
         "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "fp8_e4m3" if w.fp8 else "bf16", "data": "synthetic",
         "config": {"workload": w.name, "E": w.E, "d": w.d, "ffn": w.I, "T": w.T, "top_k": w.k,
-                   "routed_rows": w.R, "routing": w.routing, "tile_variant": args.variant},
+                   "routed_rows": w.R, "routing": w.routing, "tile_variant": args.variant,
+                   "tail_tiles_cut_along_k": not args.no_split},
         "roofline": roofline,
+        "stage_timing": "ms = per launch with several launches inside one HIP event pair on the launch stream (5 for the "
+                        "GEMMs; the row kernels' ms_back_to_back with 10), comparable with a profiler's kernel durations; "
+                        "ms_single_launch / the row kernels' ms = one launch inside its own event pair, which also holds "
+                        "the events' own packets and the launch's ramp-up on an idle chip",
         "stages": {k: {kk: (round(vv, 5) if isinstance(vv, float) else vv) for kk, vv in v.items()} for k, v in stages.items()},
     }
     if not args.no_cpu:

@@ -260,7 +260,8 @@ void gmm_tile256_kernel(const GmmArgs p) {
                 constexpr int kWaveFloats = TM * TN;
                 unsigned long long *mine = (unsigned long long *)(p.partials + ((size_t)(cur_split_tile * plan.split + cur_part) * NW + wave) * kWaveFloats);
 #pragma unroll
-                for (int i = 0; i < FM; ++i)
+                for (int i = 0; i < FM; ++i) {
+                    if (kGuard && i >= nfr) continue;      // wave-uniform: row fragments without a valid row stay out
 #pragma unroll
                     for (int j = 0; j < FN; ++j)
 #pragma unroll
@@ -269,6 +270,7 @@ void gmm_tile256_kernel(const GmmArgs p) {
                                                          ((unsigned long long)__float_as_uint(acc[i][j][2 * x + 1]) << 32);
                             __hip_atomic_store(mine + ((i * FN + j) * 2 + x) * 64 + lane, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                         }
+                }
                 __atomic_signal_fence(__ATOMIC_SEQ_CST);
                 DMOE_WAIT_VMCNT(0);
                 __atomic_signal_fence(__ATOMIC_SEQ_CST);
@@ -287,7 +289,8 @@ void gmm_tile256_kernel(const GmmArgs p) {
                     for (int k = 0; k < plan.split; ++k) {
                         unsigned long long *src = (unsigned long long *)(p.partials + ((size_t)(cur_split_tile * plan.split + k) * NW + wave) * kWaveFloats);
 #pragma unroll
-                        for (int i = 0; i < FM; ++i)
+                        for (int i = 0; i < FM; ++i) {
+                            if (kGuard && i >= nfr) continue;
 #pragma unroll
                             for (int j = 0; j < FN; ++j)
 #pragma unroll
@@ -296,6 +299,7 @@ void gmm_tile256_kernel(const GmmArgs p) {
                                     acc[i][j][2 * x] += __uint_as_float((unsigned int)v);
                                     acc[i][j][2 * x + 1] += __uint_as_float((unsigned int)(v >> 32));
                                 }
+                        }
                     }
                 }
             }

@@ -66,6 +66,11 @@ void gmm_tile256_kernel(const GmmArgs p) {
     const WorkPlan plan = plan_work((long long)s_tile_start[E] * n_tiles, G, S_all,
                                     p.arrive != nullptr ? p.partial_bytes / kPieceBytes : 0, kWsArriveCount / NW);
     const long long total = plan.items;
+    // A launch whose m-tiles are less than half full on average (a decode-sized batch) streams weights, and what its loop
+    // does besides is what the stream has to overlap with: its short tiles read only the row fragments that hold a valid
+    // row and run every stage as one phase of all wavefronts (one barrier) instead of two alternating ones.  Elsewhere
+    // short tiles keep the schedule of the full tiles they share operands with.
+    const bool lean = 2ll * s_row_start[E] < (long long)s_tile_start[E] * kDM;
     const uint32_t pitch = (uint32_t)p.K * 2;
     const uint32_t smem_addr = lds_addr(smem);
     const int streams = (G % kXcds == 0) ? kXcds : 1;
@@ -156,14 +161,17 @@ void gmm_tile256_kernel(const GmmArgs p) {
     };
 
     bf16x8 fa[FM], fb[FN];
-    auto load_operands = [&](int s) {
+    // `lim`: row fragments to read (wave-uniform; FM for a full tile); a wavefront without a valid row reads nothing
+    auto load_operands = [&](int s, int lim) {
         const char *tA = smem + (s % kStages) * kStage;
         const char *tB = tA + kStageA;
 #pragma unroll
         for (int i = 0; i < FM; ++i) {
+            if (i >= lim) break;
             const u32x4 x = *(const u32x4 *)(tA + fa_base + i * (16 * 64));
             __builtin_memcpy(&fa[i], &x, 16);
         }
+        if (lim <= 0) return;
 #pragma unroll
         for (int j = 0; j < FN; ++j) {
             if constexpr (TRANS_B) {
@@ -203,6 +211,10 @@ void gmm_tile256_kernel(const GmmArgs p) {
 
         auto run_tile = [&](auto guard_tag) {
             constexpr bool kGuard = decltype(guard_tag)::value;
+            // Alternating phases of the two halves of the workgroup, or one phase per stage: the same for every wavefront
+            // of the workgroup (they share the barriers), so the one-phase form needs a tile in which every wavefront runs
+            // this guarded build: at most 7 row fragments in the upper half, none in the lower.
+            const bool kAlt = !(kGuard && lean && cur_rows_e <= (FM - 1) * 16);
             f32x4 acc[FM][FN];
 #pragma unroll
             for (int i = 0; i < FM; ++i)
@@ -223,12 +235,17 @@ void gmm_tile256_kernel(const GmmArgs p) {
                     if constexpr (kRefill) DMOE_WAIT_VMCNT((kStages - 2) * kLoads);
                     else wait_ahead(ahead);
                 };
-                load_operands(s);
+                load_operands(s, kAlt ? FM : nfr);
                 if constexpr (kRefill) static_for<0, kLoads>([&](auto c) { issue_copy(s + kStages - 1, c); });
-                if (next && wm == 1) landed();
-                __builtin_amdgcn_sched_barrier(0);
-                __syncthreads();
-                __builtin_amdgcn_sched_barrier(0);
+                if (kAlt) {
+                    if (next && wm == 1) landed();
+                    __builtin_amdgcn_sched_barrier(0);
+                    __syncthreads();
+                    __builtin_amdgcn_sched_barrier(0);
+                } else {
+                    // one phase: the slot refilled above was read by everyone before the barrier that ended the stage before
+                    if (next) landed();
+                }
                 __builtin_amdgcn_s_setprio(1);
                 static_for<0, FM>([&](auto i_tag) {
                     constexpr int i = decltype(i_tag)::value;
@@ -238,12 +255,12 @@ void gmm_tile256_kernel(const GmmArgs p) {
                         acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fb[j], fa[i], acc[i][j], 0, 0, 0);
                 });
                 __builtin_amdgcn_s_setprio(0);
-                if (next && wm == 0) landed();
+                if (kAlt && next && wm == 0) landed();
                 __builtin_amdgcn_sched_barrier(0);
                 __syncthreads();
                 __builtin_amdgcn_sched_barrier(0);
             };
-            if (wm == 1) __syncthreads();                  // the late half
+            if (kAlt && wm == 1) __syncthreads();          // the late half
             int s = 0;
             stage(0, std::false_type{}, (S - 2 < kStages - 2 ? S - 2 : kStages - 2), S > 1);
             for (s = 1; s + kStages - 1 < S; ++s) stage(s, std::true_type{}, 0, true);
@@ -251,7 +268,7 @@ void gmm_tile256_kernel(const GmmArgs p) {
                 const int left = S - 1 - s;
                 stage(s, std::false_type{}, left - 1 < kStages - 2 ? left - 1 : kStages - 2, left > 0);
             }
-            if (wm == 0) __syncthreads();
+            if (kAlt && wm == 0) __syncthreads();
 
             bool finish = true;
             if (cur_part >= 0) {

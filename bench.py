@@ -216,6 +216,19 @@ def main() -> int:
                 fn()
         return _event_ms(many, max(2, it // 2), plug=plug)[0] / n
 
+    def rotating_ms(call, inputs, n=12):
+        """ms per launch when n launches follow each other inside one event interval, each on the next of several
+        copies of the input and into the next of as many output buffers (the ring keeps the outputs alive, so the
+        allocator hands out different blocks): more than the 256 MB Infinity Cache in all, so that no launch finds the
+        bytes of the one before it in a cache"""
+        ring = [None] * len(inputs)
+        def many():
+            for i in range(n):
+                ring[i % len(inputs)] = call(inputs[i % len(inputs)])
+        return _event_ms(many, max(2, it // 2), plug=plug)[0] / n
+
+    n_sets = max(4, int(768e6 // ((w.T + w.R) * w.d * 2)) + 1)      # at least 768 MB under the timing loop
+    n_sets = min(n_sets, 64)
     ms, _ = _event_ms(lambda: memory.permute_tokens_cuda(x, mappings), it, plug=plug)
     # "GB/s" counts a read and a write per routed row; the kernel reads a token once for its k copies ("moved")
     moved = (w.T + w.R) * w.d * 2 + 8.0 * w.R
@@ -223,6 +236,11 @@ def main() -> int:
                          "GB/s_moved": moved / ms / 1e6, "frac_hbm_moved": moved / ms / 1e6 / PEAK_HBM_GBS}
     ms = sustained_ms(lambda: memory.permute_tokens_cuda(x, mappings))
     stages["permute"].update({"ms_back_to_back": ms, "frac_hbm_moved_back_to_back": moved / ms / 1e6 / PEAK_HBM_GBS})
+    xs = [x] + [x.clone() for _ in range(n_sets - 1)]
+    ms = rotating_ms(lambda xi: memory.permute_tokens_cuda(xi, mappings), xs)
+    stages["permute"].update({"ms_rotating_buffers": ms, "frac_hbm_moved_rotating_buffers": moved / ms / 1e6 / PEAK_HBM_GBS,
+                              "rotating_sets": n_sets})
+    del xs
     if w.fp8:
         xq, xs = gg.quantize_rows(permuted)
         h = gg.gmm_fp8_swiglu(xq, xs, layer.w13_q, layer.w13_scale, batch_sizes)
@@ -270,6 +288,23 @@ def main() -> int:
     stages["combine"] = {"ms": ms, "GB/s": w.combine_bytes / ms / 1e6, "frac_hbm": w.combine_bytes / ms / 1e6 / PEAK_HBM_GBS}
     ms = sustained_ms(lambda: memory.combine_tokens(y, mappings, gates))
     stages["combine"].update({"ms_back_to_back": ms, "frac_hbm_back_to_back": w.combine_bytes / ms / 1e6 / PEAK_HBM_GBS})
+    ys = [y] + [y.clone() for _ in range(n_sets - 1)]
+    ms = rotating_ms(lambda yi: memory.combine_tokens(yi, mappings, gates), ys)
+    stages["combine"].update({"ms_rotating_buffers": ms, "frac_hbm_rotating_buffers": w.combine_bytes / ms / 1e6 / PEAK_HBM_GBS,
+                              "rotating_sets": n_sets})
+    # yardstick, not part of the path: torch's device copy of the [R, d] rows over the same rotating buffers
+    copy_bytes = 2.0 * w.R * w.d * 2
+    dsts = [torch.empty_like(yi) for yi in ys]
+    slot = [0]
+    def copy_next(_):
+        i = slot[0] = (slot[0] + 1) % len(ys)
+        dsts[i].copy_(ys[i - 1])
+        return None
+    ms = rotating_ms(copy_next, ys)
+    stages["library_device_copy"] = {"ms_rotating_buffers": ms, "GB/s": copy_bytes / ms / 1e6, "frac_hbm": copy_bytes / ms / 1e6 / PEAK_HBM_GBS,
+                                     "what": "torch copy_ of [R, d] bf16 rows (read + write) over the rotating buffers: what a plain copy "
+                                             "kernel sustains on this chip on bytes that no cache holds"}
+    del ys, dsts
 
     # algorithmic bytes of the two GEMM launches: weights of the experts that have rows, the rows in, the rows out
     ws = 1 if w.fp8 else 2
@@ -306,7 +341,9 @@ def main() -> int:
         "stage_timing": "ms = per launch with several launches inside one HIP event pair on the launch stream (5 for the "
                         "GEMMs; the row kernels' ms_back_to_back with 10), comparable with a profiler's kernel durations; "
                         "ms_single_launch / the row kernels' ms = one launch inside its own event pair, which also holds "
-                        "the events' own packets and the launch's ramp-up on an idle chip",
+                        "the events' own packets and the launch's ramp-up on an idle chip; the row kernels' "
+                        "ms_rotating_buffers = 12 launches back to back over rotating_sets copies of the input and as many "
+                        "output buffers (more than the Infinity Cache holds)",
         "stages": {k: {kk: (round(vv, 5) if isinstance(vv, float) else vv) for kk, vv in v.items()} for k, v in stages.items()},
     }
     if not args.no_cpu:

@@ -270,6 +270,18 @@ def main() -> int:
                   else f"dmoe::gmm_kernel<{tile}, 256, .., swiglu, bf16>") + " (gate-up projection with fused SiLU*mul)"
     up_flops = 2.0 * w.R * w.d * 2 * w.I
     down_flops = 2.0 * w.R * w.I * w.d
+    if w.fp8:
+        # yardstick, not part of the path: the vendor library's dense fp8 GEMM (torch._scaled_mm) of the gate-up launch's
+        # flop count, one expert's quantised weights, unit scales; skipped (with the reason) where torch refuses it
+        try:
+            one = torch.ones((), dtype=torch.float32, device=dev)
+            wq_t = layer.w13_q[0].t()                     # [d, 2I] column-major view of the K-contiguous [2I, d] weights
+            lib_ms, _ = gemm_ms(lambda: torch._scaled_mm(xq, wq_t, scale_a=one, scale_b=one, out_dtype=torch.bfloat16))
+            stages["library_dense_gemm"] = {"ms": lib_ms, "TFLOP/s": up_flops / lib_ms / 1e9, "frac_mfma": up_flops / lib_ms / 1e9 / peak,
+                                            "what": "torch._scaled_mm (hipBLASLt, fp8 e4m3 x fp8 e4m3 -> bf16, unit scales) on [R, d] x "
+                                                    "[d, 2I]: the flop count of the gate-up launch as one dense GEMM"}
+        except Exception as err:   # noqa: BLE001 - a yardstick must not break the bench
+            stages["library_dense_gemm"] = {"ms": None, "what": f"torch._scaled_mm refused: {str(err)[:160]}"}
     if not w.fp8:
         # yardstick, not part of the path: the vendor library's dense GEMM of the gate-up launch's flop count
         # ([R, d] x [d, 2I], one expert's weights, no SiLU*mul), timed the same way on the same box

@@ -189,6 +189,29 @@ def test_gmm_weights_beyond_32bit_offsets(trans_b):
     assert torch.isfinite(out.float()).all()
 
 
+@pytest.mark.parametrize("trans_b", [False, True])
+@pytest.mark.parametrize("K", [2048, 96])
+def test_gmm_decode_sized_batch_on_tall_tiles(trans_b, K):
+    # 256-row tiles that are less than half full on average: tiles of at most 112 rows run one phase per stage with
+    # reads of their valid row fragments only, the taller ones of the same launch (113, 130 rows: the lower half of the
+    # wavefronts has rows too) keep the two alternating phases; an empty expert between them
+    announce(test="gmm_decode_tall_tiles", trans_b=trans_b, K=K)
+    gg.set_tile_variant(7)
+    sizes = torch.tensor([5, 40, 100, 112, 113, 130, 0, 60], dtype=torch.int64)
+    E, R, N = len(sizes), int(sizes.sum()), 1024
+    a = _rand((R, K), 71)
+    b = _rand((E, K, N), 72, std=0.05)
+    w13 = _rand((E, K, 2 * N), 73, std=0.05)
+    up = ffn.gmm(a, w13, sizes, out_dtype=torch.float32)
+    ref_h = torch.nn.functional.silu(up[:, :N]) * up[:, N:]
+    bd = b.transpose(1, 2).contiguous() if trans_b else b
+    wd = w13.transpose(1, 2).contiguous() if trans_b else w13
+    out = gg.gmm(a.to(dev()), bd.to(dev()), sizes, trans_b=trans_b)
+    assert max_rel_err(out, ffn.gmm(a, b, sizes)) <= TOL_BF16
+    h = gg.gmm_swiglu(a.to(dev()), wd.to(dev()), sizes, trans_b=trans_b)
+    assert max_rel_err(h, ref_h) <= TOL_BF16
+
+
 @pytest.mark.parametrize("variant", [0, 5, 6, 7])
 @pytest.mark.parametrize("K", [32, 64, 96])
 def test_gmm_few_stages(variant, K):

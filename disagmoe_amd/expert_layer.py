@@ -57,7 +57,9 @@ class ExpertWorker:
     the bookkeeping lists are reordered and the layer stepped) followed by ``run(layer_id, x)`` (device:
     uploads from the staging into the static buffers, FFN, scale + return permute in one kernel).
     ``run`` touches no Python-side data, so it can be recorded into a HIP graph and replayed after each
-    ``stage`` of a batch of the same row count.
+    ``stage`` of a batch of the same row count; a replay reads the pinned staging when it executes, so the
+    caller waits for it (the graph's stream) before staging the next batch.  In eager use ``stage``
+    waits by itself for the uploads of the step before.
 
     ``reference_weight_pairing=True`` reproduces the reference's scale exactly: it builds the weight
     tensor from the lists AFTER ``sort_by_prefill_order`` has reordered them (:715, then :726) and
@@ -84,9 +86,11 @@ class ExpertWorker:
         self._host_mappings = torch.zeros(n, dtype=torch.int64, pin_memory=True)
         self._host_weights = torch.zeros(n, dtype=torch.bfloat16, pin_memory=True)
         self.h2d_stream = torch.cuda.Stream(device=dev)
-        self._uploaded = torch.cuda.Event()       # the staging has been read: it may be rewritten
+        self._uploaded = torch.cuda.Event()       # the staged mapping and weights have been read: they may be rewritten
+        self._sizes_uploaded = torch.cuda.Event() # the staged batch sizes have been read (they travel on the step's stream)
         self._consumed = torch.cuda.Event()       # the static buffers have been read: they may be rewritten
         self._uploaded.record(torch.cuda.current_stream(dev))
+        self._sizes_uploaded.record(torch.cuda.current_stream(dev))
         self._consumed.record(torch.cuda.current_stream(dev))
         self._rows = 0
         self._overflow = None                     # (mappings, weights) of a batch beyond max_batch_size
@@ -104,6 +108,7 @@ class ExpertWorker:
             weights = list(meta.topk_weights) if self.reference_weight_pairing else own_weights
             assert len(weights) == rows, f"{len(weights)} top-k weights for {rows} rows"
         self._uploaded.synchronize()              # the previous step's uploads have left the staging
+        self._sizes_uploaded.synchronize()
         self._host_batch_sizes.copy_(torch.tensor(sizes, dtype=torch.int64))
         if rows <= self.max_batch_size:
             self._host_mappings[:rows].copy_(torch.tensor(mapping, dtype=torch.int64))
@@ -125,6 +130,8 @@ class ExpertWorker:
         dev = self.device
         cur = torch.cuda.current_stream(dev)
         self.static_batch_sizes.copy_(self._host_batch_sizes, non_blocking=True)
+        if not torch.cuda.is_current_stream_capturing():
+            self._sizes_uploaded.record(cur)
         if self._overflow is not None:
             mappings = self._overflow[0].to(dev, non_blocking=True)
             weights = self._overflow[1].to(dev, non_blocking=True) if self._overflow[1] is not None else None

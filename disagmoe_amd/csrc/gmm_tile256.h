@@ -244,6 +244,8 @@ void gmm_tile256_kernel(const GmmArgs p) {
                 load_operands(s, kAlt ? FM : nfr);
                 if constexpr (kRefill) static_for<0, kLoads>([&](auto c) { issue_copy(s + kStages - 1, c); });
                 if (kAlt) {
+                    // the guarded build has its operands in registers before the barrier (see load_operands)
+                    if constexpr (kGuard) __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0)
                     if (next && wm == 1) landed();
                     __builtin_amdgcn_sched_barrier(0);
                     __syncthreads();

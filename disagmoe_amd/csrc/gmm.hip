@@ -97,13 +97,15 @@ void gmm_kernel(const GmmArgs p) {
     __shared__ long long s_item;
     const int streams = (G % kXcds == 0) ? kXcds : 1;
     unsigned int draw = 0;
-    if (tid == 0) draw = sched_draw(p.sched, streams);
+    if (tid == 0) draw = sched_draw(p.sched, streams);       // always one draw ahead
+    bool first = true;                                       // the first item needs no draw (see sched_item)
     for (;;) {
-        if (tid == 0) s_item = sched_item(draw, streams);
+        if (tid == 0) s_item = first ? (long long)blockIdx.x : sched_item(draw, streams);
         __syncthreads();
         const long long q = s_item;
         if (q >= total) break;
-        if (tid == 0) draw = sched_draw(p.sched, streams);   // next item; the round trip hides behind this tile
+        if (tid == 0 && !first) draw = sched_draw(p.sched, streams);   // next item; the round trip hides behind this tile
+        first = false;
         const TileCoord tc = decode_tile<BM>(item_order(q, G, total), n_tiles, E, s_tile_start, s_row_start);
         const int e = tc.e, nt = tc.nt, row0 = tc.row0, rows_e = tc.rows_e;
         const int n0 = nt * BNO;                               // first output column

@@ -59,8 +59,11 @@ static_assert(kWsArriveOffset + kWsArriveCount * sizeof(unsigned int) == DMOE_GM
 __device__ __forceinline__ unsigned int sched_draw(SchedSlot *slot, int streams) {
     return atomicAdd(&slot->next[streams == 1 ? 0 : (blockIdx.x % kXcds)], 1u);
 }
+// A workgroup's first item is its own number (no draw, so the first tile does not wait for an atomic's round trip);
+// the draws number the items behind those gridDim.x.
 __device__ __forceinline__ long long sched_item(unsigned int j, int streams) {
-    return streams == 1 ? (long long)j : (long long)j * kXcds + (blockIdx.x % kXcds);
+    return streams == 1 ? (long long)j + gridDim.x
+                        : ((long long)j + gridDim.x / kXcds) * kXcds + (blockIdx.x % kXcds);
 }
 // Called once per workgroup after its last draw; the last caller of the launch clears the counters.
 __device__ __forceinline__ void sched_finish(SchedSlot *slot) {

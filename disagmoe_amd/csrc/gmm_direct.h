@@ -264,13 +264,8 @@ void gmm_direct_kernel(const GmmArgs p) {
     // ---- first work item ----
     unsigned int draw = 0;
     const bool drawer = tid == (NP ? NW * 64 : 0);
-    if (drawer) {
-        draw = sched_draw(p.sched, streams);
-        s_item = sched_item(draw, streams);
-        draw = sched_draw(p.sched, streams);   // always one draw ahead: its round trip hides behind a tile
-    }
-    __syncthreads();
-    long long q = s_item;
+    if (drawer) draw = sched_draw(p.sched, streams);   // always one draw ahead: its round trip hides behind a tile
+    long long q = blockIdx.x;                          // the first item needs no draw (see sched_item)
     if (q < total) {
         if (NP == 0 || cw >= 0) {
             open_tile(q);

@@ -387,7 +387,7 @@ void gmm_kernel(const GmmArgs p) {
             }
         }
     }
-    sched_finish(p.sched);
+    sched_finish(p.sched, tid == 0, draw, streams, total);
 }
 
 template <int BM, int BN, int WM, int WN, bool TRANS_B, bool SWIGLU, bool FP8>

@@ -41,8 +41,8 @@ struct GmmArgs {
 // j = 0, 1, 2, ... and works on item q = 8 j + x, which keeps the items that share operand tiles on one
 // L2 (see item_order) exactly as a static stride would, while a slow tile no longer holds up the tiles
 // queued behind it.  The counters of a launch live in device memory that is zero when the launch starts
-// (the caller's state block, or the library's own slot of the launch's stream); the last workgroup
-// to finish clears them again.  Launches that may overlap in time must not share them.
+// (the caller's state block, or the library's own slot of the launch's stream); the workgroup that
+// makes a counter's last draw clears it again (sched_finish).  Launches that may overlap in time must not share them.
 struct SchedSlot {
     unsigned int next[kXcds];
     unsigned int done;
@@ -65,20 +65,21 @@ __device__ __forceinline__ long long sched_item(unsigned int j, int streams) {
     return streams == 1 ? (long long)j + gridDim.x
                         : ((long long)j + gridDim.x / kXcds) * kXcds + (blockIdx.x % kXcds);
 }
-// Called once per workgroup after its last draw; the last caller of the launch clears the counters.
-__device__ __forceinline__ void sched_finish(SchedSlot *slot) {
-    if (threadIdx.x == 0) {
-        __threadfence();
-        const unsigned int before = atomicAdd(&slot->done, 1u);
-        if (before == gridDim.x - 1) {
-            // cleared with the same kind of operation the counters are advanced with, so that the clear is
-            // seen wherever the next launch's draws are performed
-#pragma unroll
-            for (int i = 0; i < kXcds; ++i) atomicExch(&slot->next[i], 0u);
-            atomicExch(&slot->done, 0u);
-            __threadfence();
-        }
-    }
+// Called once per workgroup when its draw has come back past the end of the work (`draw` is that value, held by the
+// workgroup's drawing thread).  Every workgroup makes one draw more than it works on drawn items, so a counter hands
+// out exactly (its XCD's drawn items) + (its XCD's workgroups) values in a launch: whoever holds the last of them knows
+// that nobody will draw from that counter again and sets it back to zero for the next launch: no count of finished
+// workgroups, no atomic to wait for at the end of a launch.
+__device__ __forceinline__ void sched_finish(SchedSlot *slot, bool drawer, unsigned int draw, int streams, long long total) {
+    if (!drawer) return;
+    const int x = streams == 1 ? 0 : (int)(blockIdx.x % kXcds);
+    const long long wgs = streams == 1 ? (long long)gridDim.x : (long long)(gridDim.x / kXcds);
+    // drawn items of this counter: j >= 0 with sched_item(j) < total
+    long long drawn = streams == 1 ? total - wgs : (total - x + kXcds - 1) / kXcds - wgs;
+    if (drawn < 0) drawn = 0;
+    // cleared with the same kind of operation the counter is advanced with, so that the clear is seen wherever the
+    // next launch's draws are performed
+    if ((long long)draw == drawn + wgs - 1) atomicExch(&slot->next[x], 0u);
 }
 
 // ---- the last, partly filled round of tiles ----------------------------------------------------------

@@ -296,7 +296,7 @@ void gmm_direct_kernel(const GmmArgs p) {
                     issue_prologue();
                 }
             }
-            sched_finish(p.sched);
+            sched_finish(p.sched, drawer, draw, streams, total);
             return;
         }
     }
@@ -651,7 +651,7 @@ void gmm_direct_kernel(const GmmArgs p) {
         if constexpr (NP == 0) next_item();
         else if (q < total) locate_tile(q);
     }
-    sched_finish(p.sched);
+    sched_finish(p.sched, drawer, draw, streams, total);
 }
 
 template <int kDM, int NW, int WM, bool TRANS_B, bool SWIGLU, bool FP8, int NP = 0>

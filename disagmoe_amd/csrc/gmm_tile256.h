@@ -382,7 +382,7 @@ void gmm_tile256_kernel(const GmmArgs p) {
             issue_prologue();
         }
     }
-    sched_finish(p.sched);
+    sched_finish(p.sched, drawer, draw, streams, total);
 }
 
 template <bool TRANS_B, bool SWIGLU>

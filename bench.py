@@ -39,7 +39,8 @@ def _tile_rows(w) -> int:
     cus = torch.cuda.get_device_properties(0).multi_processor_count
     n_tiles = (w.I + 127) // 128
     tile = 256
-    if w.fp8 or (w.R // 256 + (w.E + 1) // 2) * n_tiles < cus:
+    est256, est128 = (w.R // 256 + (w.E + 1) // 2) * n_tiles, (w.R // 128 + (w.E + 1) // 2) * n_tiles
+    if w.fp8 or (est256 < cus and not est128 > cus):
         avg = w.R // w.E
         tile = 64 if avg <= 64 else (128 if avg <= 160 else 256)
         while tile > 64 and (w.R // tile + (w.E + 1) // 2) * n_tiles * 2 < cus:

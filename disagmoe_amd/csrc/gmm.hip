@@ -483,8 +483,11 @@ static int launch_by_rows(const GmmArgs &args, hipStream_t stream) {
     // the rows per expert on average decide, and a size that would leave more than half of the CUs without a tile is
     // halved (small problems: latency counts).
     const long long n_tiles = ((SWIGLU ? args.N / 2 : args.N) + (SWIGLU ? 127 : 255)) / (SWIGLU ? 128 : 256);
+    // ... and where 128-row tiles would need a second round for what 256-row tiles do in one (a small batch on few
+    // experts: 176 half-filled tall tiles instead of 264: 12 % off that launch).
     int tile_rows = 256;
-    if (FP8 || (args.rows / 256 + (args.E + 1) / 2) * n_tiles < device_cus()) {
+    const long long est256 = (args.rows / 256 + (args.E + 1) / 2) * n_tiles, est128 = (args.rows / 128 + (args.E + 1) / 2) * n_tiles;
+    if (FP8 || (est256 < device_cus() && !(est128 > device_cus()))) {
         tile_rows = avg <= 64 ? 64 : (avg <= 160 ? 128 : 256);
         while (tile_rows > 64 && (args.rows / tile_rows + (args.E + 1) / 2) * n_tiles * 2 < device_cus()) tile_rows /= 2;
     }

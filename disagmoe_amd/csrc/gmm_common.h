@@ -97,6 +97,8 @@ struct WorkPlan {
 };
 constexpr int kMaxSplit = 8;
 constexpr int kMaxWholeRounds = 3;
+constexpr int kMinPieceStagesIdle = 24;   // ... unless the launch has fewer tiles than workgroups: the pieces then run
+                                          // on compute units that would have nothing to do
 constexpr int kMinPieceStages = 88;   // shorter pieces lose to their own overhead (measured: tiles of 44 and 128 stages
                                       // lose when cut, tiles of 448 stages cut in 4 or 5 gain 7 - 11 %)
 
@@ -114,12 +116,14 @@ __device__ __host__ __forceinline__ WorkPlan plan_work(long long tiles, int G, i
     const long long whole_cost = stages + 8;
     long long best_cost = whole_cost;
     for (int p = 2; p <= kMaxSplit; ++p) {
-        if (rem * p > max_pieces || stages / p < kMinPieceStages) break;
+        if (rem * p > max_pieces || stages / p < (tiles < G ? kMinPieceStagesIdle : kMinPieceStages)) break;
         const long long rounds = (rem * p + G - 1) / G;
         const long long cost = rounds * ((stages + p - 1) / p + 20) + 4 + 4 * p;
         if (cost < best_cost) { best = p; best_cost = cost; }
     }
-    if (best == 1 || best_cost * 100 > 92 * whole_cost) return w;
+    // the estimate flatters short pieces (measured: 0.79 of a whole tile's time where it says 0.69), so they have to
+    // promise more
+    if (best == 1 || best_cost * 100 > (tiles < G ? 85 : 92) * whole_cost) return w;
     w.split = best; w.rem = (int)rem; w.whole = tiles - rem; w.items = w.whole + rem * best;
     return w;
 }

@@ -665,8 +665,12 @@ static int launch_direct_one(const GmmArgs &args, hipStream_t stream) {
     const int n_out = SWIGLU ? args.N / 2 : args.N;
     const long long n_tiles = (n_out + BNO - 1) / BNO;
     const long long m_tiles_max = args.rows / kDM + args.E;
+    // a launch that may cut its tiles along K (workspace, K long enough for two pieces) can use more workgroups than
+    // it has tiles
+    long long pieces = m_tiles_max * n_tiles;
+    if (args.arrive != nullptr && args.K / (FP8 ? 64 : kDK) >= 2 * kMinPieceStagesIdle) pieces *= kMaxSplit;
     long long grid = (long long)device_cus();
-    if (m_tiles_max * n_tiles < grid) grid = m_tiles_max * n_tiles;
+    if (pieces < grid) grid = pieces;
     if (grid < 1) grid = 1;
     grid = (grid + kXcds - 1) / kXcds * kXcds;   // whole rows of XCDs: the tile order is XCD-aware only then
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3((NW + NP) * 64), lds, stream, args);

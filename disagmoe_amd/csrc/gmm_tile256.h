@@ -397,7 +397,7 @@ static int launch_tile256_one(const GmmArgs &args, hipStream_t stream) {
     const long long m_tiles_max = args.rows / 256 + args.E;
     // a launch that may cut its tiles along K (workspace, long K) can use more workgroups than it has tiles
     long long pieces = m_tiles_max * n_tiles;
-    if (args.arrive != nullptr && args.K / kDK >= 2 * kMinPieceStages) pieces *= kMaxSplit;
+    if (args.arrive != nullptr && args.K / kDK >= 2 * kMinPieceStagesIdle) pieces *= kMaxSplit;
     long long grid = (long long)device_cus();
     if (pieces < grid) grid = pieces;
     if (grid < 1) grid = 1;

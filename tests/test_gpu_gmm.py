@@ -254,8 +254,8 @@ def _expected_split(sizes, tile_rows, n_out, swiglu, K, workspace_bytes):
     n_tiles = -(-n_out // (128 if swiglu else 256))
     rows, E = int(sum(sizes)), len(sizes)
     pieces = (rows // tile_rows + E) * n_tiles
-    if tile_rows == 256 and K // 32 >= 2 * 88:
-        pieces *= 8                                  # the 256-row launch may use more workgroups than it has tiles
+    if K // 32 >= 2 * 24:
+        pieces *= 8                                  # a launch that may cut tiles may use more workgroups than it has tiles
     grid = -(-max(min(cus, pieces), 1) // 8) * 8
     tiles = sum(-(-n // tile_rows) for n in sizes) * n_tiles
     stages, rem = K // 32, tiles % grid
@@ -265,14 +265,15 @@ def _expected_split(sizes, tile_rows, n_out, swiglu, K, workspace_bytes):
     if tiles // grid > 3:
         return 1
     best, best_cost = 1, stages + 8
+    min_piece = 24 if tiles < grid else 88           # pieces may be short where they run on compute units that have no tile
     for p in range(2, 9):
-        if rem * p > max_pieces or stages // p < 88:
+        if rem * p > max_pieces or stages // p < min_piece:
             break
         rounds = -(-rem * p // grid)
         cost = rounds * (-(-stages // p) + 20) + 4 + 4 * p
         if cost < best_cost:
             best, best_cost = p, cost
-    return 1 if best == 1 or best_cost * 100 > 92 * (stages + 8) else best
+    return 1 if best == 1 or best_cost * 100 > (85 if tiles < grid else 92) * (stages + 8) else best
 
 
 @pytest.mark.parametrize("variant", [5, 6, 7, 0])

@@ -123,7 +123,7 @@ __device__ __host__ __forceinline__ WorkPlan plan_work(long long tiles, int G, i
     }
     // the estimate flatters short pieces (measured: 0.79 of a whole tile's time where it says 0.69), so they have to
     // promise more
-    if (best == 1 || best_cost * 100 > (tiles < G ? 85 : 92) * whole_cost) return w;
+    if (best == 1 || best_cost * 100 > (stages / best < kMinPieceStages ? 85 : 92) * whole_cost) return w;
     w.split = best; w.rem = (int)rem; w.whole = tiles - rem; w.items = w.whole + rem * best;
     return w;
 }

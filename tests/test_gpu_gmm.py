@@ -273,7 +273,7 @@ def _expected_split(sizes, tile_rows, n_out, swiglu, K, workspace_bytes):
         cost = rounds * (-(-stages // p) + 20) + 4 + 4 * p
         if cost < best_cost:
             best, best_cost = p, cost
-    return 1 if best == 1 or best_cost * 100 > (85 if tiles < grid else 92) * (stages + 8) else best
+    return 1 if best == 1 or best_cost * 100 > (85 if stages // best < 88 else 92) * (stages + 8) else best
 
 
 @pytest.mark.parametrize("variant", [5, 6, 7, 0])

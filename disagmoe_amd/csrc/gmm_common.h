@@ -256,5 +256,6 @@ __device__ __forceinline__ WorkItem decode_item(long long q, int G, const WorkPl
 
 int launch_direct_bf16(const GmmArgs &args, int tile_rows, bool trans_b, bool swiglu, hipStream_t stream);
 int launch_direct_fp8(const GmmArgs &args, int tile_rows, bool swiglu, hipStream_t stream);
+int launch_tile256_fp8(const GmmArgs &args, bool swiglu, hipStream_t stream);
 
 }  // namespace dmoe

@@ -185,6 +185,39 @@ def test_gmm_fp8_few_stages(variant, K):
         gg.set_tile_variant(0)
 
 
+@pytest.mark.parametrize("swiglu", [False, True])
+@pytest.mark.parametrize("K,N,sizes", [
+    (128, 256, [256, 0, 1, 255, 257]),                 # one k-step; full, empty, 1-row, 255-row tiles and a 1-row last tile
+    (1152, 520, [300, 17, 0, 513, 128]),               # 9 k-steps; a ragged last n-tile
+    (3200, 512, [500, 0, 290]),                        # fewer tiles than compute units, long K: cut along K in uneven pieces
+])
+def test_gmm_fp8_tile_of_whole_lines(K, N, sizes, swiglu):
+    """The 256-row fp8 tile whose copies fetch whole 128-byte lines (K % 128 == 0; variant 7 picks 256-row tiles)."""
+    announce(test="gmm_fp8_tile_of_whole_lines", K=K, N=N, sizes=sizes, swiglu=swiglu)
+    gg.set_tile_variant(7)
+    try:
+        E, R = len(sizes), sum(sizes)
+        n_w = 2 * N if swiglu else N
+        g = torch.Generator().manual_seed(K + N)
+        a = torch.randn(R, K, generator=g).to(torch.bfloat16)
+        w = (torch.randn(E, K, n_w, generator=g) * 0.05).to(torch.bfloat16)
+        bs = torch.tensor(sizes, dtype=torch.int64)
+        aq, a_s = fp8.quantize_rows(a)
+        wq, w_s = fp8.quantize_weight_channels(w)
+        run = gg.gmm_fp8_swiglu if swiglu else gg.gmm_fp8
+        out = run(aq.to(dev()), a_s.to(dev()), wq.to(dev()), w_s.to(dev()), bs)
+        exact = ffn.gmm(fp8.dequantize_rows(aq, a_s, torch.float32), fp8.dequantize_weight(wq, w_s, torch.float32), bs,
+                        out_dtype=torch.float32)
+        if swiglu:
+            exact = torch.nn.functional.silu(exact[:, :N]) * exact[:, N:]
+        assert out.shape == exact.shape
+        assert max_rel_err(out, exact) <= 1e-2, max_rel_err(out, exact)
+        again = run(aq.to(dev()), a_s.to(dev()), wq.to(dev()), w_s.to(dev()), bs)
+        assert torch.equal(out, again)                 # pieces are summed in a fixed order
+    finally:
+        gg.set_tile_variant(0)
+
+
 @pytest.mark.parametrize("T,d,k,E", [(1, 16, 1, 1), (37, 1024, 2, 8), (100, 2048, 6, 64), (64, 6144, 2, 8), (5, 16384, 2, 4),
                                      (3, 32768, 2, 2)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])

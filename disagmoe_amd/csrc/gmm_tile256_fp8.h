@@ -109,22 +109,30 @@ void gmm_tile256_fp8_kernel(const GmmArgs p) {
 #pragma unroll
         for (int i = 0; i < CB; ++i) b_off[i] = (uint32_t)b_col((i * NW + wave) * 8 + kc_row) * pitch + kc_chunk * 16;
     };
-    // the copies of k-step t of the item
-    auto issue_step = [&](int t) {
+    // The copies of k-step t of the item, in two groups by when their place in LDS is free.  The B tile and the A rows
+    // of row fragments 0 - 3 of either half of the tile (this wavefront's blocks 0 and 2) are read in the first memory
+    // phase of a k-step, the A rows of row fragments 4 - 7 (blocks 1 and 3) in the second.
+    auto issue_early = [&](int t) {
         const uint32_t lds = smem_addr + (t % kBufs) * kBuf + wave * 1024;
         const uint64_t k_off = (uint64_t)t * kStepK;
-        static_for<0, CA>([&](auto i_tag) {
-            constexpr int i = decltype(i_tag)::value;
-            copy_g2lds_16<i * kBlock>(a_off[i], a_base + k_off, lds);
-        });
         static_for<0, CB>([&](auto i_tag) {
             constexpr int i = decltype(i_tag)::value;
             copy_g2lds_16<kBufA + i * kBlock>(b_off[i], b_exp + k_off, lds);
         });
+        copy_g2lds_16<0 * kBlock>(a_off[0], a_base + k_off, lds);
+        copy_g2lds_16<2 * kBlock>(a_off[2], a_base + k_off, lds);
     };
+    auto issue_late = [&](int t) {
+        const uint32_t lds = smem_addr + (t % kBufs) * kBuf + wave * 1024;
+        const uint64_t k_off = (uint64_t)t * kStepK;
+        copy_g2lds_16<1 * kBlock>(a_off[1], a_base + k_off, lds);
+        copy_g2lds_16<3 * kBlock>(a_off[3], a_base + k_off, lds);
+    };
+    constexpr int kEarly = CB + 2, kLate = 2;
     auto issue_prologue = [&]() {
-        issue_step(0);
-        if (T > 1) issue_step(1);
+        issue_early(0);
+        issue_late(0);
+        if (T > 1) { issue_early(1); issue_late(1); }
     };
 
     i32x8 fa[FM / 2], fb[FN];
@@ -158,15 +166,24 @@ void gmm_tile256_fp8_kernel(const GmmArgs p) {
 #pragma unroll
                 for (int j = 0; j < FN; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-            // k-step 0 has landed (k-step 1 may be in flight)
-            if (T > 1) DMOE_WAIT_VMCNT(kCopies); else DMOE_WAIT_VMCNT(0);
+            // the early group of k-step 0 has landed (its late group and k-step 1 may be in flight)
+            if (T > 1) DMOE_WAIT_VMCNT(kLate + kEarly + kLate); else DMOE_WAIT_VMCNT(kLate);
             __syncthreads();
             // Phases of k-step t, for the early half of the wavefronts (the late half one phase later): memory a (the B
-            // fragments, row fragments 0 - 3; from t = 1 on the copies of k-step t + 1, whose slots k-step t - 1 has left:
-            // the late half read them last in its memory phase b, one barrier ago), matrix a, memory b (row fragments
-            // 4 - 7), matrix b.  Before the barrier that closes the late half's memory b every wavefront has waited for
-            // its copies of k-step t + 1, the only ones in flight.
-            auto half_step = [&](int t, auto h_tag, bool refill, bool next) {
+            // fragments, row fragments 0 - 3), matrix a, memory b (row fragments 4 - 7), matrix b.  What memory a reads is
+            // free once the late half has left its memory a, so memory b of k-step t issues the early group of k-step
+            // t + 2 into it, and memory a of k-step t + 1 the late group of k-step t + 2 (the prologue stands in for the
+            // first ones): a copy is in flight for a k-step and a half.  A wavefront's copies complete in the order early(t),
+            // late(t), early(t + 1), ...; before the barrier that lets the early half into memory a of k-step t + 1 every
+            // wavefront has waited for its early(t + 1), behind which it has issued late(t + 1) and early(t + 2), and
+            // before the barrier that lets it into memory b of k-step t for its late(t), behind which early(t + 1) and late(t + 1).
+            auto landed_early = [&](int t) {   // early(t + 1), at the end of k-step t
+                if (t + 2 < T) DMOE_WAIT_VMCNT(kLate + kEarly); else DMOE_WAIT_VMCNT(kLate);
+            };
+            auto landed_late = [&](int t) {    // late(t), in the middle of k-step t
+                if (t + 1 < T) DMOE_WAIT_VMCNT(kEarly + kLate); else DMOE_WAIT_VMCNT(0);
+            };
+            auto half_step = [&](int t, auto h_tag, bool next) {
                 constexpr int h = decltype(h_tag)::value;
                 const char *base = smem + (t % kBufs) * kBuf;
                 if (h == 0) {
@@ -175,8 +192,12 @@ void gmm_tile256_fp8_kernel(const GmmArgs p) {
                 }
 #pragma unroll
                 for (int i = 0; i < FM / 2; ++i) fa[i] = read32(base, fa_base, (h * (FM / 2) + i) * (16 * kStepK));
-                if (h == 0 && refill) issue_step(t + 1);
-                if (h == 1 && next && wm == 1) DMOE_WAIT_VMCNT(0);
+                if (h == 0 && t >= 1 && next) issue_late(t + 1);
+                if (h == 1 && t + 2 < T) issue_early(t + 2);
+                if (wm == 1) {
+                    if (h == 0) landed_late(t);
+                    else if (next) landed_early(t);
+                }
                 __builtin_amdgcn_sched_barrier(0);
                 __syncthreads();
                 __builtin_amdgcn_sched_barrier(0);
@@ -190,16 +211,18 @@ void gmm_tile256_fp8_kernel(const GmmArgs p) {
                                                                                      0, 0, 0, 0, 0, 0);
                 });
                 __builtin_amdgcn_s_setprio(0);
-                if (h == 1 && next && wm == 0) DMOE_WAIT_VMCNT(0);
+                if (wm == 0) {
+                    if (h == 0) landed_late(t);
+                    else if (next) landed_early(t);
+                }
                 __builtin_amdgcn_sched_barrier(0);
                 __syncthreads();
                 __builtin_amdgcn_sched_barrier(0);
             };
             if (wm == 1) __syncthreads();                  // the late half
             for (int t = 0; t < T; ++t) {
-                const bool refill = t >= 1 && t + 1 < T;
-                half_step(t, std::integral_constant<int, 0>{}, refill, t + 1 < T);
-                half_step(t, std::integral_constant<int, 1>{}, refill, t + 1 < T);
+                half_step(t, std::integral_constant<int, 0>{}, t + 1 < T);
+                half_step(t, std::integral_constant<int, 1>{}, t + 1 < T);
             }
             if (wm == 0) __syncthreads();
 

@@ -255,8 +255,10 @@ def main() -> int:
         stages["permute_quantize"] = {"ms": pq_ms, "GB/s": (2.0 * w.T + w.R) * w.d / pq_ms / 1e6}   # bytes actually moved
         peak = PEAK_FP8_TFLOPS
         tile = _tile_rows(w)
-        # mirrors the dispatch of launch_by_rows (csrc/gmm.hip): the global-to-LDS kernel takes whole 64-k stages
+        # mirrors the dispatch of launch_by_rows (csrc/gmm.hip) and launch_direct_fp8: the global-to-LDS kernels take
+        # whole 64-k stages, the 256-row tile of whole 128-byte lines whole 128-k steps
         kernel = (f"dmoe::gmm_kernel<{tile}, 256, .., swiglu, fp8>" if w.d % 64
+                  else "dmoe::gmm_tile256_fp8_kernel<swiglu>" if tile == 256 and w.d % 128 == 0
                   else f"dmoe::gmm_direct_kernel<{tile}, .., swiglu, fp8>") + " (gate-up projection with fused SiLU*mul)"
     else:
         h = gg.gmm_swiglu(permuted, layer.w13_weight, batch_sizes, **gemm_state)

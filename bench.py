@@ -30,7 +30,7 @@ PEAK_FP8_TFLOPS = 5000.0
 MEASURED_TRAFFIC = {"C2": (4.089e9, "profiles/expert_layer_c2_hbm_traffic.md"),
                     "C3": (1.926e9, "profiles/expert_layer_c5_c4_c3_hbm_traffic.md"),
                     "C4": (1.495e9, "profiles/expert_layer_c5_c4_c3_hbm_traffic.md"),
-                    "C5": (13.322e9, "profiles/expert_layer_c5_c4_c3_hbm_traffic.md")}
+                    "C5": (17.893e9, "profiles/expert_layer_c5_c4_c3_hbm_traffic.md")}
 
 
 def _tile_rows(w) -> int:

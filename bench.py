@@ -40,7 +40,9 @@ def _tile_rows(w) -> int:
     n_tiles = (w.I + 127) // 128
     tile = 256
     est256, est128 = (w.R // 256 + (w.E + 1) // 2) * n_tiles, (w.R // 128 + (w.E + 1) // 2) * n_tiles
-    if w.fp8 or (est256 < cus and not est128 > cus):
+    # (the gate-up launch of the bench has a workspace: tiles may be cut along K when K / 64 >= 48)
+    tall = (w.d % 128 == 0 and est256 * (4 if w.d // 64 >= 48 else 2) >= cus) if w.fp8 else (est256 >= cus or est128 > cus)
+    if not tall:
         avg = w.R // w.E
         tile = 64 if avg <= 64 else (128 if avg <= 160 else 256)
         while tile > 64 and (w.R // tile + (w.E + 1) // 2) * n_tiles * 2 < cus:

@@ -487,7 +487,14 @@ static int launch_by_rows(const GmmArgs &args, hipStream_t stream) {
     // experts: 176 half-filled tall tiles instead of 264: 12 % off that launch).
     int tile_rows = 256;
     const long long est256 = (args.rows / 256 + (args.E + 1) / 2) * n_tiles, est128 = (args.rows / 128 + (args.E + 1) / 2) * n_tiles;
-    if (FP8 || (est256 < device_cus() && !(est128 > device_cus()))) {
+    // fp8: the 256-row tile copies whole 128-byte lines (gmm_tile256_fp8.h) and streams weights a third faster than the
+    // smaller tiles, which copy half lines (decode-sized batch on the 8x7B shapes: 4.1 against 3.2 TB/s); it is taken
+    // wherever its tiles fill half of the CUs
+    // (a quarter, where the launch may cut its tiles along a long K to fill the rest)
+    const bool may_cut = args.arrive != nullptr && args.K / 64 >= 2 * kMinPieceStagesIdle;
+    const bool tall = FP8 ? (args.K % 128 == 0 && est256 * (may_cut ? 4 : 2) >= device_cus())
+                          : (est256 >= device_cus() || est128 > device_cus());
+    if (!tall) {
         tile_rows = avg <= 64 ? 64 : (avg <= 160 ? 128 : 256);
         while (tile_rows > 64 && (args.rows / tile_rows + (args.E + 1) / 2) * n_tiles * 2 < device_cus()) tile_rows /= 2;
     }

@@ -218,6 +218,31 @@ def test_gmm_fp8_tile_of_whole_lines(K, N, sizes, swiglu):
         gg.set_tile_variant(0)
 
 
+@pytest.mark.parametrize("swiglu", [False, True])
+def test_gmm_fp8_decode_sized_batch_on_many_experts(swiglu):
+    """64 experts with 0 .. 20 rows each: the default tile choice gives such a launch the 256-row tile of whole lines
+    (its tiles fill more than half of the compute units), every tile of it a few rows high."""
+    announce(test="gmm_fp8_decode_sized_batch_on_many_experts", swiglu=swiglu)
+    E, K, N = 64, 2048, 1408
+    g = torch.Generator().manual_seed(64)
+    sizes = torch.randint(0, 21, (E,), generator=g)
+    sizes[3] = 0
+    sizes[E - 1] = 0
+    R = int(sizes.sum())
+    n_w = 2 * N if swiglu else N
+    a = torch.randn(R, K, generator=g).to(torch.bfloat16)
+    w = (torch.randn(E, K, n_w, generator=g) * 0.05).to(torch.bfloat16)
+    aq, a_s = fp8.quantize_rows(a)
+    wq, w_s = fp8.quantize_weight_channels(w)
+    run = gg.gmm_fp8_swiglu if swiglu else gg.gmm_fp8
+    out = run(aq.to(dev()), a_s.to(dev()), wq.to(dev()), w_s.to(dev()), sizes)
+    exact = ffn.gmm(fp8.dequantize_rows(aq, a_s, torch.float32), fp8.dequantize_weight(wq, w_s, torch.float32), sizes,
+                    out_dtype=torch.float32)
+    if swiglu:
+        exact = torch.nn.functional.silu(exact[:, :N]) * exact[:, N:]
+    assert max_rel_err(out, exact) <= 1e-2, max_rel_err(out, exact)
+
+
 @pytest.mark.parametrize("T,d,k,E", [(1, 16, 1, 1), (37, 1024, 2, 8), (100, 2048, 6, 64), (64, 6144, 2, 8), (5, 16384, 2, 4),
                                      (3, 32768, 2, 2)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])

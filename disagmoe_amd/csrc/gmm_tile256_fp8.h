@@ -37,7 +37,6 @@ void gmm_tile256_fp8_kernel(const GmmArgs p) {
     constexpr int kBuf = kBufA + kBufB;                  // 64 KiB
     constexpr int kBufs = 2;
     constexpr int CA = kDM / (8 * NW), CB = kDN / (8 * NW);   // copies (8 rows of 128 B each) per wavefront per k-step
-    constexpr int kCopies = CA + CB;
     constexpr int kBlock = NW * 1024;
     constexpr int BNO = SWIGLU ? kDN / 2 : kDN;
     static_assert(CA == 4 && CB == 4, "copies per k-step");

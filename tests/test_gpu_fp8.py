@@ -188,6 +188,8 @@ def test_gmm_fp8_few_stages(variant, K):
 @pytest.mark.parametrize("swiglu", [False, True])
 @pytest.mark.parametrize("K,N,sizes", [
     (128, 256, [256, 0, 1, 255, 257]),                 # one k-step; full, empty, 1-row, 255-row tiles and a 1-row last tile
+    (256, 264, [40, 0, 300]),                          # two k-steps: the prologue's copies are all there are
+    (384, 264, [100, 0, 257]),                         # three k-steps: one refill
     (1152, 520, [300, 17, 0, 513, 128]),               # 9 k-steps; a ragged last n-tile
     (3200, 512, [500, 0, 290]),                        # fewer tiles than compute units, long K: cut along K in uneven pieces
 ])

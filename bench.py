@@ -33,23 +33,6 @@ MEASURED_TRAFFIC = {"C2": (4.089e9, "profiles/expert_layer_c2_hbm_traffic.md"),
                     "C5": (17.893e9, "profiles/expert_layer_c5_c4_c3_hbm_traffic.md")}
 
 
-def _tile_rows(w) -> int:
-    """Tile rows the gate-up launch gets: mirrors launch_by_rows (csrc/gmm.hip)."""
-    import torch
-    cus = torch.cuda.get_device_properties(0).multi_processor_count
-    n_tiles = (w.I + 127) // 128
-    tile = 256
-    est256, est128 = (w.R // 256 + (w.E + 1) // 2) * n_tiles, (w.R // 128 + (w.E + 1) // 2) * n_tiles
-    # (the gate-up launch of the bench has a workspace: tiles may be cut along K when K / 64 >= 48)
-    tall = (w.d % 128 == 0 and est256 * (4 if w.d // 64 >= 48 else 2) >= cus) if w.fp8 else (est256 >= cus or est128 > cus)
-    if not tall:
-        avg = w.R // w.E
-        tile = 64 if avg <= 64 else (128 if avg <= 160 else 256)
-        while tile > 64 and (w.R // tile + (w.E + 1) // 2) * n_tiles * 2 < cus:
-            tile //= 2
-    return tile
-
-
 def _event_ms(fn, iters: int, warmup: int = 2, plug=None):
     """Average duration of ``fn`` in ms, HIP events on the current stream (the one
     the kernels are launched on).  ``plug`` is device work of a few ms enqueued first:
@@ -77,7 +60,7 @@ def _cpu_baseline(w, x, ids, gates, layer, budget_s: float = 12.0):
     import torch
     from oracle import cpu_path
     # the threads the environment grants this process: OMP_NUM_THREADS where it is set (a GPU box shares its host
-    # cores between its GPUs), every core otherwise
+    # cores between its GPUs), every core otherwise; the host's own core count is reported beside it
     cores = torch.get_num_threads()
     w13 = layer.w13_weight.detach().cpu()
     w2 = layer.w2_weight.detach().cpu()
@@ -99,7 +82,7 @@ def _cpu_baseline(w, x, ids, gates, layer, budget_s: float = 12.0):
             break
     times.sort()
     dt = times[len(times) // 2]
-    return {"value": n / dt, "unit": "tokens/s", "cores": cores, "kind": "port",
+    return {"value": n / dt, "unit": "tokens/s", "cores": cores, "host_cpu_count": os.cpu_count(), "kind": "port",
             "sample": f"first {n} of {w.T} tokens ({n * w.k} routed rows) through all {w.E} experts' full weights, "
                       f"median of {len(times)} passes, {dt:.2f} s each, {spent:.1f} s of CPU work in all; "
                       f"bf16 storage, torch CPU matmul (fp32 accumulate)"}
@@ -152,12 +135,12 @@ def main() -> int:
         layer.w2_weight = torch.nn.Parameter(w2, requires_grad=False)
         layer.enable_cache = False
         layer.gmm_cache_max_batch_size = 0
-    # state block and workspace of the layer's launches, as MoEExperts.create_weights sets them up
-    ws_size, args_ptr = gg.get_arguments(w.E, dev)
-    gemm_state = dict(arguments_ptr=args_ptr,
-                      workspace=None if args.no_split else torch.empty([ws_size], dtype=torch.uint8, device=dev))
+    # the layer's state block (MoEExperts.create_weights) and the stream's shared workspace
     if not w.fp8:
-        layer.arguments_ptr, layer.workspace = gemm_state["arguments_ptr"], gemm_state["workspace"]
+        layer._init_gemm_state(dev)
+    gemm_state = dict(arguments_ptr=layer.arguments_ptr, workspace=None if args.no_split else gg.shared_workspace(dev))
+    if args.no_split:
+        layer._gemm_state = lambda: gemm_state
     torch.cuda.synchronize()
 
     def step():
@@ -246,35 +229,31 @@ def main() -> int:
     del xs
     if w.fp8:
         xq, xs = gg.quantize_rows(permuted)
-        h = gg.gmm_fp8_swiglu(xq, xs, layer.w13_q, layer.w13_scale, batch_sizes)
+        h = gg.gmm_fp8_swiglu(xq, xs, layer.w13_q, layer.w13_scale, batch_sizes, **gemm_state)
         hq, hs = gg.quantize_rows(h)
-        up_ms, up_single = gemm_ms(lambda: gg.gmm_fp8_swiglu(xq, xs, layer.w13_q, layer.w13_scale, batch_sizes, c=h))
+        up_ms, up_single = gemm_ms(lambda: gg.gmm_fp8_swiglu(xq, xs, layer.w13_q, layer.w13_scale, batch_sizes, c=h, **gemm_state))
         y_buf = torch.empty((w.R, w.d), dtype=torch.bfloat16, device=dev)
-        down_ms, down_single = gemm_ms(lambda: gg.gmm_fp8(hq, hs, layer.w2_q, layer.w2_scale, batch_sizes, c=y_buf))
+        down_ms, down_single = gemm_ms(lambda: gg.gmm_fp8(hq, hs, layer.w2_q, layer.w2_scale, batch_sizes, c=y_buf, **gemm_state))
         q_ms, _ = _event_ms(lambda: gg.quantize_rows(h), it)
         stages["quant_rows"] = {"ms": q_ms, "GB/s": 3.0 * w.R * w.I / q_ms / 1e6}       # the [R, I] intermediate
         pq_ms, _ = _event_ms(lambda: memory.permute_quantize(x, mappings), it)
         stages["permute_quantize"] = {"ms": pq_ms, "GB/s": (2.0 * w.T + w.R) * w.d / pq_ms / 1e6}   # bytes actually moved
         peak = PEAK_FP8_TFLOPS
-        tile = _tile_rows(w)
-        # mirrors the dispatch of launch_by_rows (csrc/gmm.hip) and launch_direct_fp8: the global-to-LDS kernels take
-        # whole 64-k stages, the 256-row tile of whole 128-byte lines whole 128-k steps
-        kernel = (f"dmoe::gmm_kernel<{tile}, 256, .., swiglu, fp8>" if w.d % 64
-                  else "dmoe::gmm_tile256_fp8_kernel<swiglu>" if tile == 256 and w.d % 128 == 0
-                  else f"dmoe::gmm_direct_kernel<{tile}, .., swiglu, fp8>") + " (gate-up projection with fused SiLU*mul)"
     else:
         h = gg.gmm_swiglu(permuted, layer.w13_weight, batch_sizes, **gemm_state)
         up_ms, up_single = gemm_ms(lambda: gg.gmm_swiglu(permuted, layer.w13_weight, batch_sizes, c=h, **gemm_state))
         y_buf = torch.empty((w.R, w.d), dtype=torch.bfloat16, device=dev)
         down_ms, down_single = gemm_ms(lambda: gg.gmm(h, layer.w2_weight, batch_sizes, c=y_buf, **gemm_state))
         peak = PEAK_BF16_TFLOPS
-        tile = _tile_rows(w)
-        direct = w.d % 32 == 0
-        kernel = (("dmoe::gmm_tile256_kernel<[K,N] weights, swiglu>" if tile == 256 else
-                   f"dmoe::gmm_direct_kernel<{tile}, .., [K,N] weights, swiglu, bf16>") if direct
-                  else f"dmoe::gmm_kernel<{tile}, 256, .., swiglu, bf16>") + " (gate-up projection with fused SiLU*mul)"
     up_flops = 2.0 * w.R * w.d * 2 * w.I
     down_flops = 2.0 * w.R * w.I * w.d
+    # what the library launches for the two GEMMs, by its own account (kernel, tile rows, workgroups, tiles cut along K)
+    ws_bytes = 0 if args.no_split else gemm_state["workspace"].numel()
+    sizes_host = batch_sizes.cpu()
+    plan_up = gg.launch_plan(w.R, w.E, w.d, w.I, swiglu=True, fp8=w.fp8, workspace_bytes=ws_bytes, batch_sizes=sizes_host)
+    plan_down = gg.launch_plan(w.R, w.E, w.I, w.d, swiglu=False, fp8=w.fp8, workspace_bytes=ws_bytes, batch_sizes=sizes_host)
+    kernel = (f"{plan_up['kernel']} ({'fp8 e4m3' if w.fp8 else 'bf16, [K, N] weights'}, tiles of {plan_up['tile_rows']} rows, "
+              f"{plan_up['workgroups']} workgroups of {plan_up['wavefronts']} wavefronts): gate-up projection with fused SiLU*mul")
     if w.fp8:
         # yardstick, not part of the path: the vendor library's dense fp8 GEMM (torch._scaled_mm) of the gate-up launch's
         # flop count, one expert's quantised weights, unit scales; skipped (with the reason) where torch refuses it
@@ -308,8 +287,10 @@ def main() -> int:
                                              "what": "the same library call on one expert's share of the rows, [R/E, d] x [d, 2I]: what a "
                                                      "loop of E library launches would run at"}
         del one_c
-    stages["gemm_gate_up"] = {"ms": up_ms, "ms_single_launch": up_single, "TFLOP/s": up_flops / up_ms / 1e9, "frac_mfma": up_flops / up_ms / 1e9 / peak}
-    stages["gemm_down"] = {"ms": down_ms, "ms_single_launch": down_single, "TFLOP/s": down_flops / down_ms / 1e9, "frac_mfma": down_flops / down_ms / 1e9 / peak}
+    stages["gemm_gate_up"] = {"ms": up_ms, "ms_single_launch": up_single, "TFLOP/s": up_flops / up_ms / 1e9, "frac_mfma": up_flops / up_ms / 1e9 / peak,
+                              "launch": plan_up}
+    stages["gemm_down"] = {"ms": down_ms, "ms_single_launch": down_single, "TFLOP/s": down_flops / down_ms / 1e9, "frac_mfma": down_flops / down_ms / 1e9 / peak,
+                           "launch": plan_down}
     stages["gemm_total"] = {"ms": up_ms + down_ms, "TFLOP/s": w.gemm_flops / (up_ms + down_ms) / 1e9,
                             "frac_mfma": w.gemm_flops / (up_ms + down_ms) / 1e9 / peak}
     y = layer.forward(w.R, permuted, batch_sizes)

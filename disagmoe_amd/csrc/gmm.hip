@@ -25,6 +25,7 @@
 namespace dmoe {
 
 constexpr int kRowBytes = 128;     // bytes of K per tile row in LDS
+constexpr int kDK32 = 32;          // k per stage of the global -> LDS bf16 kernels (gmm_direct.h)
 
 // XOR applied to the 16-byte chunk index of a 128-byte LDS row.  Its period is
 // 16 rows, so fragment rows 32 apart differ by a constant.
@@ -393,18 +394,12 @@ void gmm_kernel(const GmmArgs p) {
 template <int BM, int BN, int WM, int WN, bool TRANS_B, bool SWIGLU, bool FP8>
 static int launch_one(const GmmArgs &args, hipStream_t stream) {
     constexpr int NT = WM * WN * kWave;
-    constexpr int BNO = SWIGLU ? BN / 2 : BN;
+    static_assert(BN == 256, "launch_grid counts tiles of 256 columns");
     const size_t lds = 2 * (size_t)(BM + BN) * kRowBytes;
     auto kern = gmm_kernel<BM, BN, WM, WN, TRANS_B, SWIGLU, FP8>;
     static unsigned long long configured = 0;   // devices on which the kernel's LDS size has been raised
     DMOE_HIP(raise_dynamic_lds((const void *)kern, (int)lds, &configured));
-    const int n_out = SWIGLU ? args.N / 2 : args.N;
-    const long long n_tiles = (n_out + BNO - 1) / BNO;
-    const long long m_tiles_max = args.rows / BM + args.E;  // sum of ceil(n_e / BM) never exceeds this
-    long long grid = (long long)device_cus();
-    if (m_tiles_max * n_tiles < grid) grid = m_tiles_max * n_tiles;
-    if (grid < 1) grid = 1;
-    grid = (grid + kXcds - 1) / kXcds * kXcds;   // whole rows of XCDs: the tile order is XCD-aware only then
+    const long long grid = launch_grid(args, BM, SWIGLU, 64, false, device_cus());
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NT), lds, stream, args);
     DMOE_LAUNCH_CHECK("gmm_kernel");
     return DMOE_OK;
@@ -442,9 +437,19 @@ static int own_slot(hipStream_t stream, SchedSlot **out) {
     int slot = -1;
     for (int i = 0; i < used[dev]; ++i)
         if (table[dev][i].stream == stream) { slot = i; break; }
+    if (slot < 0 && used[dev] == kOwnSlots) {
+        // every slot has had a stream: take over one whose stream has no work pending (its last launch has returned the
+        // counters to zero) or no longer exists
+        for (int i = 0; i < kOwnSlots && slot < 0; ++i) {
+            const hipError_t busy = hipStreamQuery(table[dev][i].stream);
+            if (busy != hipSuccess) (void)hipGetLastError();
+            if (busy != hipErrorNotReady) slot = i;
+        }
+        DMOE_REQUIRE(slot >= 0, DMOE_ERR_WORKSPACE,
+                     "grouped GEMM: %d streams on device %d have launches without a state block pending; pass one", kOwnSlots, dev);
+        table[dev][slot] = Entry{dev, stream};
+    }
     if (slot < 0) {
-        DMOE_REQUIRE(used[dev] < kOwnSlots, DMOE_ERR_WORKSPACE,
-                     "grouped GEMM: more than %d streams on device %d without a state block; pass one", kOwnSlots, dev);
         slot = used[dev]++;
         table[dev][slot] = Entry{dev, stream};
     }
@@ -466,60 +471,88 @@ static int bind_state(GmmArgs &args, void *state, void *workspace, size_t worksp
     return DMOE_OK;
 }
 
-template <bool TRANS_B, bool SWIGLU, bool FP8>
-static int launch_by_rows(const GmmArgs &args, hipStream_t stream) {
-    // the host does not know how the rows split over the experts
-    const long long avg = args.rows / (args.E > 0 ? args.E : 1);
-    switch (g_variant) {
-        case 1: return launch_one<256, 256, 2, 2, TRANS_B, SWIGLU, FP8>(args, stream);
-        case 2: return launch_one<64, 256, 1, 4, TRANS_B, SWIGLU, FP8>(args, stream);
-        case 3: return launch_one<128, 256, 1, 4, TRANS_B, SWIGLU, FP8>(args, stream);
-        case 4: return launch_one<256, 256, 2, 4, TRANS_B, SWIGLU, FP8>(args, stream);
-        default: break;
-    }
-    // Tile rows.  Every m-tile streams its 256 columns of the weights through the CU whatever its rows, so fewer, taller
-    // tiles move fewer bytes (decode-sized batches: 8 tiles of 256 rows instead of 12 of 64 on the Zipf batch, 10 % off the
-    // gate-up launch) and a tile's empty row fragments cost no MFMAs: 256 rows wherever such tiles fill the CUs.  Else
-    // the rows per expert on average decide, and a size that would leave more than half of the CUs without a tile is
-    // halved (small problems: latency counts).
-    const long long n_tiles = ((SWIGLU ? args.N / 2 : args.N) + (SWIGLU ? 127 : 255)) / (SWIGLU ? 128 : 256);
-    // ... and where 128-row tiles would need a second round for what 256-row tiles do in one (a small batch on few
-    // experts: 176 half-filled tall tiles instead of 264: 12 % off that launch).
-    int tile_rows = 256;
-    const long long est256 = (args.rows / 256 + (args.E + 1) / 2) * n_tiles, est128 = (args.rows / 128 + (args.E + 1) / 2) * n_tiles;
-    // fp8: the 256-row tile copies whole 128-byte lines (gmm_tile256_fp8.h) and streams weights a third faster than the
-    // smaller tiles, which copy half lines (decode-sized batch on the 8x7B shapes: 4.1 against 3.2 TB/s); it is taken
-    // wherever its tiles fill half of the CUs
-    // (a quarter, where the launch may cut its tiles along a long K to fill the rest)
-    const bool may_cut = args.arrive != nullptr && args.K / 64 >= 2 * kMinPieceStagesIdle;
-    const bool tall = FP8 ? (args.K % 128 == 0 && est256 * (may_cut ? 4 : 2) >= device_cus())
-                          : (est256 >= device_cus() || est128 > device_cus());
-    if (!tall) {
-        tile_rows = avg <= 64 ? 64 : (avg <= 160 ? 128 : 256);
-        while (tile_rows > 64 && (args.rows / tile_rows + (args.E + 1) / 2) * n_tiles * 2 < device_cus()) tile_rows /= 2;
-    }
-    if (g_variant >= 5) tile_rows = g_variant == 5 ? 64 : (g_variant == 6 ? 128 : 256);   // direct kernel, fixed tile rows
-    if constexpr (!FP8) {
-        // global -> LDS direct path: whole stages of 32 k, 32-bit offsets inside one expert's weights
-        if (args.K % 32 == 0 && (long long)args.K * args.N * 2 < (1ll << 32))
-            return launch_direct_bf16(args, tile_rows, TRANS_B, SWIGLU, stream);
+// Kernel, tile rows and grid of a launch, from what the host knows (the shapes, not how the rows split over the experts).
+// The one place where that is decided: launch_by_rows dispatches on the result and dmoe_gmm_plan reports it.
+static GmmLaunch choose_launch(const GmmArgs &args, bool swiglu, bool fp8) {
+    const int cus = device_cus();
+    GmmLaunch L{};
+    if (g_variant >= 1 && g_variant <= 4) {   // test hook: the register-staged kernel with a fixed tile
+        L.kernel = kKernelStaged;
+        L.tile_rows = g_variant == 2 ? 64 : (g_variant == 3 ? 128 : 256);
+        L.waves = g_variant == 4 ? 8 : 4;
     } else {
-        if (args.K % 64 == 0 && (long long)args.K * args.N < (1ll << 32))
-            return launch_direct_fp8(args, tile_rows, SWIGLU, stream);
+        // Tile rows.  Every m-tile streams its 256 columns of the weights through the CU whatever its rows, so fewer,
+        // taller tiles move fewer bytes (decode-sized batches: 8 tiles of 256 rows instead of 12 of 64 on a Zipf batch of
+        // 512 rows, 10 % off the gate-up launch) and a tile's empty row fragments cost no MFMAs: 256 rows wherever such
+        // tiles fill the CUs, and where 128-row tiles would need a second round for what 256-row tiles do in one (a
+        // small batch on few experts: 176 half-filled tall tiles instead of 264: 12 % off that launch).  Else the rows
+        // per expert on average decide, and a size that would leave more than half of the CUs without a tile is halved
+        // (small problems: latency counts).
+        const long long avg = args.rows / (args.E > 0 ? args.E : 1);
+        const long long n_tiles = ((swiglu ? args.N / 2 : args.N) + (swiglu ? 127 : 255)) / (swiglu ? 128 : 256);
+        const long long est256 = (args.rows / 256 + (args.E + 1) / 2) * n_tiles, est128 = (args.rows / 128 + (args.E + 1) / 2) * n_tiles;
+        // fp8: the 256-row tile copies whole 128-byte lines (gmm_tile256_fp8.h) and streams weights a third faster than
+        // the smaller tiles, which copy half lines (decode-sized batch, K 4096, N 28672: 4.1 against 3.2 TB/s); it is
+        // taken wherever its tiles fill half of the CUs (a quarter, where the launch may cut its tiles along a long K
+        // to fill the rest)
+        const bool may_cut = args.arrive != nullptr && args.K / 64 >= 2 * kMinPieceStagesIdle;
+        const bool tall = fp8 ? (args.K % 128 == 0 && est256 * (may_cut ? 4 : 2) >= cus) : (est256 >= cus || est128 > cus);
+        int tile_rows = 256;
+        if (!tall) {
+            tile_rows = avg <= 64 ? 64 : (avg <= 160 ? 128 : 256);
+            while (tile_rows > 64 && (args.rows / tile_rows + (args.E + 1) / 2) * n_tiles * 2 < cus) tile_rows /= 2;
+        }
+        if (g_variant >= 5) tile_rows = g_variant == 5 ? 64 : (g_variant == 6 ? 128 : 256);   // test hook: fixed tile rows
+        L.tile_rows = tile_rows;
+        // global -> LDS kernels: whole stages (32 k of bf16, 64 of fp8), 32-bit offsets inside one expert's weights
+        const bool direct = fp8 ? (args.K % 64 == 0 && (long long)args.K * args.N < (1ll << 32))
+                                : (args.K % 32 == 0 && (long long)args.K * args.N * 2 < (1ll << 32));
+        if (!direct) {
+            L.kernel = kKernelStaged;
+            L.waves = tile_rows == 256 ? 8 : 4;
+        } else if (tile_rows == 256 && !fp8) {
+            L.kernel = kKernelTile256; L.waves = 8;
+        } else if (tile_rows == 256 && args.K % 128 == 0) {
+            L.kernel = kKernelTile256Fp8; L.waves = 8;   // whole k-steps of 128: the tile that copies whole 128-byte lines
+        } else {
+            // fp8 tiles of 256 rows on 4 wavefronts would need 256 accumulator + 96 operand registers per lane: 8 wavefronts
+            L.kernel = kKernelDirect;
+            L.waves = tile_rows == 256 ? 8 : (tile_rows == 64 && !fp8 ? 6 : 4);
+        }
     }
-    if (tile_rows == 64) return launch_one<64, 256, 1, 4, TRANS_B, SWIGLU, FP8>(args, stream);
-    if (tile_rows == 128) return launch_one<128, 256, 1, 4, TRANS_B, SWIGLU, FP8>(args, stream);
-    return launch_one<256, 256, 2, 4, TRANS_B, SWIGLU, FP8>(args, stream);
+    L.stage_k = fp8 ? 64 : (L.kernel == kKernelStaged ? 64 : kDK32);
+    L.may_cut = L.kernel != kKernelStaged;
+    L.grid = launch_grid(args, L.tile_rows, swiglu, L.stage_k, L.may_cut, cus);
+    return L;
 }
 
-static int check_gmm(const char *who, const void *a, const void *b, const void *c, const int64_t *bs, int64_t rows,
-                     int E, int64_t K, int64_t N, int align) {
+template <bool TRANS_B, bool SWIGLU, bool FP8>
+static int launch_by_rows(const GmmArgs &args, hipStream_t stream) {
+    const GmmLaunch L = choose_launch(args, SWIGLU, FP8);
+    if (L.kernel == kKernelStaged) {
+        if (L.tile_rows == 64) return launch_one<64, 256, 1, 4, TRANS_B, SWIGLU, FP8>(args, stream);
+        if (L.tile_rows == 128) return launch_one<128, 256, 1, 4, TRANS_B, SWIGLU, FP8>(args, stream);
+        if (L.waves == 4) return launch_one<256, 256, 2, 2, TRANS_B, SWIGLU, FP8>(args, stream);
+        return launch_one<256, 256, 2, 4, TRANS_B, SWIGLU, FP8>(args, stream);
+    }
+    if constexpr (FP8) return launch_direct_fp8(args, L.tile_rows, SWIGLU, stream);
+    else return launch_direct_bf16(args, L.tile_rows, TRANS_B, SWIGLU, stream);
+}
+
+static int check_shape(const char *who, int64_t rows, int E, int64_t K, int64_t N, int align) {
     DMOE_REQUIRE(rows >= 0 && rows < (1ll << 31), DMOE_ERR_SHAPE, "%s: rows=%lld outside [0, 2^31)", who, (long long)rows);
     DMOE_REQUIRE(E > 0 && E <= kMaxGroups, DMOE_ERR_SHAPE, "%s: E=%d outside [1, %d]", who, E, kMaxGroups);
     DMOE_REQUIRE(K > 0 && K < (1ll << 22) && K % align == 0, DMOE_ERR_SHAPE, "%s: K=%lld must be a positive multiple of %d",
                  who, (long long)K, align);
     DMOE_REQUIRE(N > 0 && N < (1ll << 24) && N % 8 == 0, DMOE_ERR_SHAPE, "%s: N=%lld must be a positive multiple of 8", who,
                  (long long)N);
+    return DMOE_OK;
+}
+
+static int check_gmm(const char *who, const void *a, const void *b, const void *c, const int64_t *bs, int64_t rows,
+                     int E, int64_t K, int64_t N, int align) {
+    const int rc = check_shape(who, rows, E, K, N, align);
+    if (rc != DMOE_OK) return rc;
     DMOE_REQUIRE(bs != nullptr && b != nullptr, DMOE_ERR_ARG, "%s: null pointer", who);
     DMOE_REQUIRE(rows == 0 || (a != nullptr && c != nullptr), DMOE_ERR_ARG, "%s: null pointer", who);
     return DMOE_OK;
@@ -532,6 +565,47 @@ using namespace dmoe;
 extern "C" int dmoe_gmm_tune(int variant) {
     DMOE_REQUIRE(variant >= 0 && variant <= 7, DMOE_ERR_ARG, "dmoe_gmm_tune: variant %d outside [0, 7]", variant);
     g_variant = variant;
+    return DMOE_OK;
+}
+
+// What a launch with these shapes would run (see tuning.h).  out: [0] kernel (GmmKernelId), [1] tile rows, [2] wavefronts
+// per workgroup, [3] workgroups, [4] k per stage unit; and, when the sizes are given (host memory), what the kernel
+// derives from them on the device: [5] tiles, [6] tiles cut along K, [7] pieces per cut tile, [8] work items; -1 without.
+extern "C" int dmoe_gmm_plan(const int64_t *host_batch_sizes, int64_t rows, int E, int64_t K, int64_t N, int swiglu,
+                             int dtype, size_t workspace_bytes, int64_t *out) {
+    DMOE_REQUIRE(out != nullptr, DMOE_ERR_ARG, "dmoe_gmm_plan: null output");
+    DMOE_REQUIRE(dtype == DMOE_BF16 || dtype == DMOE_FP8_E4M3, DMOE_ERR_DTYPE, "dmoe_gmm_plan: dtype %d", dtype);
+    const bool fp8 = dtype == DMOE_FP8_E4M3;
+    const int64_t n_cols = swiglu ? 2 * N : N;
+    int rc = check_shape("dmoe_gmm_plan", rows, E, K, n_cols, fp8 ? 16 : 8);
+    if (rc != DMOE_OK) return rc;
+    GmmArgs args{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, rows, E, (int)K, (int)n_cols, (int)N};
+    args.arrive = workspace_bytes > 0 ? (unsigned int *)out : nullptr;   // only tested against nullptr
+    args.partial_bytes = (long long)workspace_bytes;
+    const GmmLaunch L = choose_launch(args, swiglu != 0, fp8);
+    out[0] = L.kernel; out[1] = L.tile_rows; out[2] = L.waves; out[3] = L.grid; out[4] = L.stage_k;
+    out[5] = out[6] = out[7] = out[8] = -1;
+    if (host_batch_sizes != nullptr) {
+        long long m_tiles = 0, left = rows;
+        for (int e = 0; e < E; ++e) {
+            long long n = host_batch_sizes[e] < 0 ? 0 : host_batch_sizes[e];
+            if (n > left) n = left;
+            left -= n;
+            m_tiles += (n + L.tile_rows - 1) / L.tile_rows;
+        }
+        const long long n_tiles = (N + (swiglu ? 127 : 255)) / (swiglu ? 128 : 256);
+        WorkPlan w;
+        if (L.may_cut) {
+            const long long piece_bytes = (long long)L.tile_rows * 256 * sizeof(float);
+            // the 256-row fp8 tile counts its length in k-steps of 128 and plans in twice that many stage units
+            const int stages = (int)(L.kernel == kKernelTile256Fp8 ? 2 * (K / 128) : K / L.stage_k);
+            w = plan_work(m_tiles * n_tiles, (int)L.grid, stages, workspace_bytes > 0 ? (long long)workspace_bytes / piece_bytes : 0,
+                          kWsArriveCount / (L.waves == 6 ? 4 : L.waves));
+        } else {
+            w.tiles = w.whole = w.items = m_tiles * n_tiles; w.rem = 0; w.split = 1;
+        }
+        out[5] = w.tiles; out[6] = w.rem; out[7] = w.split; out[8] = w.items;
+    }
     return DMOE_OK;
 }
 

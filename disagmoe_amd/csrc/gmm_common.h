@@ -254,6 +254,93 @@ __device__ __forceinline__ WorkItem decode_item(long long q, int G, const WorkPl
     return it;
 }
 
+// ---- a piece of a split tile meets the others ---------------------------------------------------------
+// Every wavefront leaves its accumulators in the workspace, as [fragment][value pair][lane] so that an instruction
+// moves 512 bytes, and counts itself in at the counter of its part of the tile.  The wavefront that arrives last there,
+// of whichever piece, adds the pieces up in their order (the sum does not depend on who that is) and returns true: it
+// goes on to the epilogue.  The partial sums and the counter are written and read with accesses of device scope, which
+// go past the XCD's L2 to memory that every XCD sees: no fence has to write back or invalidate a whole L2, whose
+// other contents (the operand tiles of the compute units beside this one) stay where they are.
+// AccT: a vector of 4 or 16 floats; lim: wave-uniform, the row fragments [lim, FM) hold no valid row and stay out of
+// the workspace (every piece of a tile leaves out the same ones).
+template <int NW, int FM, int FN, typename AccT>
+__device__ __forceinline__ bool meet_pieces(AccT (&acc)[FM][FN], const GmmArgs &p, int split, int split_tile, int part,
+                                            int wave, int lane, int lim) {
+    constexpr int kPairs = (int)(sizeof(AccT) / 8);
+    constexpr size_t kWaveFloats = (size_t)FM * FN * kPairs * 2 * kWave;
+    unsigned long long *mine = (unsigned long long *)(p.partials + ((size_t)(split_tile * split + part) * NW + wave) * kWaveFloats);
+#pragma unroll
+    for (int i = 0; i < FM; ++i) {
+        if (i >= lim) continue;
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int x = 0; x < kPairs; ++x) {
+                const unsigned long long v = (unsigned long long)__float_as_uint(acc[i][j][2 * x]) |
+                                             ((unsigned long long)__float_as_uint(acc[i][j][2 * x + 1]) << 32);
+                __hip_atomic_store(mine + ((i * FN + j) * kPairs + x) * kWave + lane, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+    }
+    // the stores have reached memory before the wavefront counts itself in
+    __atomic_signal_fence(__ATOMIC_SEQ_CST);
+    __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (15 << 8));   // vmcnt(0)
+    __atomic_signal_fence(__ATOMIC_SEQ_CST);
+    unsigned int *arrived = p.arrive + split_tile * NW + wave;
+    unsigned int before = 0;
+    if (lane == 0) before = __hip_atomic_fetch_add(arrived, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    before = __builtin_amdgcn_readfirstlane(before);
+    __atomic_signal_fence(__ATOMIC_SEQ_CST);
+    if (before != (unsigned int)(split - 1)) return false;
+    if (lane == 0) __hip_atomic_store(arrived, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // as the next launch expects it
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int x = 0; x < 2 * kPairs; ++x) acc[i][j][x] = 0.f;
+    for (int k = 0; k < split; ++k) {
+        const unsigned long long *src = (const unsigned long long *)(p.partials + ((size_t)(split_tile * split + k) * NW + wave) * kWaveFloats);
+#pragma unroll
+        for (int i = 0; i < FM; ++i) {
+            if (i >= lim) continue;
+#pragma unroll
+            for (int j = 0; j < FN; ++j)
+#pragma unroll
+                for (int x = 0; x < kPairs; ++x) {
+                    const unsigned long long v = __hip_atomic_load(src + ((i * FN + j) * kPairs + x) * kWave + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    acc[i][j][2 * x] += __uint_as_float((unsigned int)v);
+                    acc[i][j][2 * x + 1] += __uint_as_float((unsigned int)(v >> 32));
+                }
+        }
+    }
+    return true;
+}
+
+// ---- the launch a problem gets (host) -------------------------------------------------------------------
+enum GmmKernelId { kKernelStaged = 0, kKernelDirect = 1, kKernelTile256 = 2, kKernelTile256Fp8 = 3 };
+struct GmmLaunch {
+    int kernel;        // GmmKernelId
+    int tile_rows;     // rows of a tile (64, 128, 256); a tile has 256 columns of b
+    int waves;         // wavefronts of a workgroup
+    int stage_k;       // k per unit of plan_work's lengths (bf16: 32; fp8: 64)
+    bool may_cut;      // the kernel cuts tiles along K when the launch has a workspace
+    long long grid;    // workgroups
+};
+// Workgroups of a persistent launch: one per compute unit, fewer when the tiles (or, where tiles may be cut along a K
+// long enough for two pieces, their pieces) do not fill them; whole rows of XCDs, the tile order is XCD-aware only then.
+// The host does not know how the rows split over the experts: rows / tile_rows + E bounds the m-tiles from above.
+inline long long launch_grid(const GmmArgs &args, int tile_rows, bool swiglu, int stage_k, bool may_cut, int cus) {
+    const int n_out = swiglu ? args.N / 2 : args.N;
+    const int bno = swiglu ? 128 : 256;
+    const long long n_tiles = (n_out + bno - 1) / bno;
+    long long pieces = (args.rows / tile_rows + args.E) * n_tiles;
+    if (may_cut && args.arrive != nullptr && args.K / stage_k >= 2 * kMinPieceStagesIdle) pieces *= kMaxSplit;
+    long long grid = cus;
+    if (pieces < grid) grid = pieces;
+    if (grid < 1) grid = 1;
+    return (grid + kXcds - 1) / kXcds * kXcds;
+}
+
 int launch_direct_bf16(const GmmArgs &args, int tile_rows, bool trans_b, bool swiglu, hipStream_t stream);
 int launch_direct_fp8(const GmmArgs &args, int tile_rows, bool swiglu, hipStream_t stream);
 int launch_tile256_fp8(const GmmArgs &args, bool swiglu, hipStream_t stream);

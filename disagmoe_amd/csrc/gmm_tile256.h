@@ -110,6 +110,9 @@ void gmm_tile256_kernel(const GmmArgs p) {
     int part = -1, split_tile = 0;
     uint64_t a_base = 0, b_exp = 0;
     uint32_t a_off[CA], b_off[CB];
+    // the expert of the item has a single m-tile: its weights pass through this workgroup once and through no other, so
+    // their copies take the non-temporal policy (wave-uniform)
+    bool b_once = false;
 
     auto b_col = [&](int slot) {
         const int rh = (SWIGLU && slot >= kDN / 2) ? slot - kDN / 2 : slot;
@@ -119,6 +122,7 @@ void gmm_tile256_kernel(const GmmArgs p) {
     auto open_tile = [&](long long q) {
         const WorkItem it = decode_item<kDM>(q, G, plan, S_all, n_tiles, E, s_tile_start, s_row_start);
         e = it.tile.e; row0 = it.tile.row0; rows_e = it.tile.rows_e; n0 = it.tile.nt * BNO;
+        b_once = __builtin_amdgcn_readfirstlane(s_tile_start[e + 1] - s_tile_start[e]) == 1;
         s_lo = it.s_lo; S = it.s_cnt; pre = S < kStages ? S : kStages;
         part = it.piece; split_tile = it.split_tile;
         a_base = to_scalar((uint64_t)(uintptr_t)p.a + (uint64_t)row0 * pitch + (uint64_t)s_lo * 64);
@@ -139,19 +143,28 @@ void gmm_tile256_kernel(const GmmArgs p) {
                 b_off[i] = (uint32_t)(i * 2 * NW + kn_k) * (uint32_t)p.N * 2 + (uint32_t)b_col(kn_chunk * 8) * 2;
         }
     };
-    auto issue_copy = [&](int s, auto c_tag) {
-        constexpr int c = decltype(c_tag)::value;
+    // the kLoads copies of this wavefront for stage s of the item: its CA blocks of A, then its CB blocks of B
+    auto issue_copies = [&](int s) {
         const uint32_t lds = smem_addr + (s % kStages) * kStage + wave * 1024;
-        if constexpr (c < CA) {
+        static_for<0, CA>([&](auto c_tag) {
+            constexpr int c = decltype(c_tag)::value;
             copy_g2lds_16<c * kBlock>(a_off[c], a_base + (uint64_t)s * 64, lds);
+        });
+        const uint64_t base = b_exp + (TRANS_B ? (uint64_t)s * 64 : (uint64_t)s * kDK * p.N * 2);
+        if (b_once) {   // one branch per stage
+            static_for<0, CB>([&](auto i_tag) {
+                constexpr int i = decltype(i_tag)::value;
+                copy_g2lds_16_nt<kStageA + i * kBlock>(b_off[i], base, lds);
+            });
         } else {
-            constexpr int i = c - CA;
-            if constexpr (TRANS_B) copy_g2lds_16<kStageA + i * kBlock>(b_off[i], b_exp + (uint64_t)s * 64, lds);
-            else copy_g2lds_16<kStageA + i * kBlock>(b_off[i], b_exp + (uint64_t)s * kDK * p.N * 2, lds);
+            static_for<0, CB>([&](auto i_tag) {
+                constexpr int i = decltype(i_tag)::value;
+                copy_g2lds_16<kStageA + i * kBlock>(b_off[i], base, lds);
+            });
         }
     };
     auto issue_prologue = [&]() {
-        for (int s = 0; s < pre; ++s) static_for<0, kLoads>([&](auto c) { issue_copy(s, c); });
+        for (int s = 0; s < pre; ++s) issue_copies(s);
     };
     auto wait_ahead = [&](int n) {   // at most n stages of this wavefront's copies outstanding
         if (n >= 3) DMOE_WAIT_VMCNT(3 * kLoads);
@@ -237,7 +250,7 @@ void gmm_tile256_kernel(const GmmArgs p) {
                     else wait_ahead(ahead);
                 };
                 load_operands(s, kAlt ? FM : nfr);
-                if constexpr (kRefill) static_for<0, kLoads>([&](auto c) { issue_copy(s + kStages - 1, c); });
+                if constexpr (kRefill) issue_copies(s + kStages - 1);
                 if (kAlt) {
                     // the guarded build has its operands in registers before the barrier (see load_operands)
                     if constexpr (kGuard) __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0)
@@ -273,57 +286,10 @@ void gmm_tile256_kernel(const GmmArgs p) {
             }
             if (kAlt && wm == 0) __syncthreads();
 
-            bool finish = true;
-            if (cur_part >= 0) {
-                // ---- a piece of a split tile (see gmm_direct.h): accumulators to the workspace past the L2, count in,
-                // the wavefront that arrives last sums the pieces in their order ----
-                constexpr int kWaveFloats = TM * TN;
-                unsigned long long *mine = (unsigned long long *)(p.partials + ((size_t)(cur_split_tile * plan.split + cur_part) * NW + wave) * kWaveFloats);
-#pragma unroll
-                for (int i = 0; i < FM; ++i) {
-                    if (kGuard && i >= nfr) continue;      // wave-uniform: row fragments without a valid row stay out
-#pragma unroll
-                    for (int j = 0; j < FN; ++j)
-#pragma unroll
-                        for (int x = 0; x < 2; ++x) {
-                            const unsigned long long v = (unsigned long long)__float_as_uint(acc[i][j][2 * x]) |
-                                                         ((unsigned long long)__float_as_uint(acc[i][j][2 * x + 1]) << 32);
-                            __hip_atomic_store(mine + ((i * FN + j) * 2 + x) * 64 + lane, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                        }
-                }
-                __atomic_signal_fence(__ATOMIC_SEQ_CST);
-                DMOE_WAIT_VMCNT(0);
-                __atomic_signal_fence(__ATOMIC_SEQ_CST);
-                unsigned int *arrived = p.arrive + cur_split_tile * NW + wave;
-                unsigned int before = 0;
-                if (lane == 0) before = __hip_atomic_fetch_add(arrived, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                before = __builtin_amdgcn_readfirstlane(before);
-                __atomic_signal_fence(__ATOMIC_SEQ_CST);
-                finish = before == (unsigned int)(plan.split - 1);
-                if (finish) {
-                    if (lane == 0) __hip_atomic_store(arrived, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-#pragma unroll
-                    for (int i = 0; i < FM; ++i)
-#pragma unroll
-                        for (int j = 0; j < FN; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-                    for (int k = 0; k < plan.split; ++k) {
-                        unsigned long long *src = (unsigned long long *)(p.partials + ((size_t)(cur_split_tile * plan.split + k) * NW + wave) * kWaveFloats);
-#pragma unroll
-                        for (int i = 0; i < FM; ++i) {
-                            if (kGuard && i >= nfr) continue;
-#pragma unroll
-                            for (int j = 0; j < FN; ++j)
-#pragma unroll
-                                for (int x = 0; x < 2; ++x) {
-                                    const unsigned long long v = __hip_atomic_load(src + ((i * FN + j) * 2 + x) * 64 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                                    acc[i][j][2 * x] += __uint_as_float((unsigned int)v);
-                                    acc[i][j][2 * x + 1] += __uint_as_float((unsigned int)(v >> 32));
-                                }
-                        }
-                    }
-                }
-            }
-            if (!finish) return;
+            // a piece of a split tile: its sums go to the workspace, and the piece that arrives last adds all of them up
+            if (cur_part >= 0 &&
+                !meet_pieces<NW>(acc, p, plan.split, cur_split_tile, cur_part, wave, lane, kGuard ? nfr : FM))
+                return;
 
             // ---- epilogue ----
             // Lane l holds, of fragment (i, j), row i * 16 + l % 16 and the 4 columns j * 16 + (l / 16) * 4 ...: 8 bytes
@@ -387,21 +353,11 @@ void gmm_tile256_kernel(const GmmArgs p) {
 
 template <bool TRANS_B, bool SWIGLU>
 static int launch_tile256_one(const GmmArgs &args, hipStream_t stream) {
-    constexpr int BNO = SWIGLU ? kDN / 2 : kDN;
     const size_t lds = (size_t)4 * (256 * kDK * 2 + kStageB);
     auto kern = gmm_tile256_kernel<TRANS_B, SWIGLU>;
     static unsigned long long configured = 0;   // devices on which the kernel's LDS size has been raised
     DMOE_HIP(raise_dynamic_lds((const void *)kern, (int)lds, &configured));
-    const int n_out = SWIGLU ? args.N / 2 : args.N;
-    const long long n_tiles = (n_out + BNO - 1) / BNO;
-    const long long m_tiles_max = args.rows / 256 + args.E;
-    // a launch that may cut its tiles along K (workspace, long K) can use more workgroups than it has tiles
-    long long pieces = m_tiles_max * n_tiles;
-    if (args.arrive != nullptr && args.K / kDK >= 2 * kMinPieceStagesIdle) pieces *= kMaxSplit;
-    long long grid = (long long)device_cus();
-    if (pieces < grid) grid = pieces;
-    if (grid < 1) grid = 1;
-    grid = (grid + kXcds - 1) / kXcds * kXcds;   // whole rows of XCDs: the tile order is XCD-aware only then
+    const long long grid = launch_grid(args, 256, SWIGLU, kDK, true, device_cus());
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(512), lds, stream, args);
     DMOE_LAUNCH_CHECK("gmm_tile256_kernel");
     return DMOE_OK;

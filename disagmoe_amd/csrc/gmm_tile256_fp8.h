@@ -227,56 +227,10 @@ void gmm_tile256_fp8_kernel(const GmmArgs p) {
             }
             if (wm == 0) __syncthreads();
 
-            bool finish = true;
-            if (cur_part >= 0) {
-                // ---- a piece of a split tile (see gmm_direct.h) ----
-                constexpr int kWaveFloats = TM * TN;
-                unsigned long long *mine = (unsigned long long *)(p.partials + ((size_t)(cur_split_tile * plan.split + cur_part) * NW + wave) * kWaveFloats);
-#pragma unroll
-                for (int i = 0; i < FM; ++i) {
-                    if (kGuard && i >= nfr) continue;      // wave-uniform: row fragments without a valid row stay out
-#pragma unroll
-                    for (int j = 0; j < FN; ++j)
-#pragma unroll
-                        for (int x = 0; x < 2; ++x) {
-                            const unsigned long long v = (unsigned long long)__float_as_uint(acc[i][j][2 * x]) |
-                                                         ((unsigned long long)__float_as_uint(acc[i][j][2 * x + 1]) << 32);
-                            __hip_atomic_store(mine + ((i * FN + j) * 2 + x) * 64 + lane, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                        }
-                }
-                __atomic_signal_fence(__ATOMIC_SEQ_CST);
-                DMOE_WAIT_VMCNT(0);
-                __atomic_signal_fence(__ATOMIC_SEQ_CST);
-                unsigned int *arrived = p.arrive + cur_split_tile * NW + wave;
-                unsigned int before = 0;
-                if (lane == 0) before = __hip_atomic_fetch_add(arrived, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                before = __builtin_amdgcn_readfirstlane(before);
-                __atomic_signal_fence(__ATOMIC_SEQ_CST);
-                finish = before == (unsigned int)(plan.split - 1);
-                if (finish) {
-                    if (lane == 0) __hip_atomic_store(arrived, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-#pragma unroll
-                    for (int i = 0; i < FM; ++i)
-#pragma unroll
-                        for (int j = 0; j < FN; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-                    for (int k = 0; k < plan.split; ++k) {
-                        unsigned long long *src = (unsigned long long *)(p.partials + ((size_t)(cur_split_tile * plan.split + k) * NW + wave) * kWaveFloats);
-#pragma unroll
-                        for (int i = 0; i < FM; ++i) {
-                            if (kGuard && i >= nfr) continue;
-#pragma unroll
-                            for (int j = 0; j < FN; ++j)
-#pragma unroll
-                                for (int x = 0; x < 2; ++x) {
-                                    const unsigned long long v = __hip_atomic_load(src + ((i * FN + j) * 2 + x) * 64 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                                    acc[i][j][2 * x] += __uint_as_float((unsigned int)v);
-                                    acc[i][j][2 * x + 1] += __uint_as_float((unsigned int)(v >> 32));
-                                }
-                        }
-                    }
-                }
-            }
-            if (!finish) return;
+            // a piece of a split tile: its sums go to the workspace, and the piece that arrives last adds all of them up
+            if (cur_part >= 0 &&
+                !meet_pieces<NW>(acc, p, plan.split, cur_split_tile, cur_part, wave, lane, kGuard ? nfr : FM))
+                return;
 
             // ---- epilogue: scales, (SiLU * up), 32 rows at a time through LDS, out by rows (see gmm_tile256.h) ----
             constexpr int RB = FNO * 32;
@@ -348,21 +302,11 @@ void gmm_tile256_fp8_kernel(const GmmArgs p) {
 
 template <bool SWIGLU>
 static int launch_tile256_fp8_one(const GmmArgs &args, hipStream_t stream) {
-    constexpr int BNO = SWIGLU ? kDN / 2 : kDN;
     const size_t lds = (size_t)2 * (256 * 128 + 256 * 128);
     auto kern = gmm_tile256_fp8_kernel<SWIGLU>;
     static unsigned long long configured = 0;   // devices on which the kernel's LDS size has been raised
     DMOE_HIP(raise_dynamic_lds((const void *)kern, (int)lds, &configured));
-    const int n_out = SWIGLU ? args.N / 2 : args.N;
-    const long long n_tiles = (n_out + BNO - 1) / BNO;
-    const long long m_tiles_max = args.rows / 256 + args.E;
-    // a launch that may cut its tiles along K (workspace, long K) can use more workgroups than it has tiles
-    long long pieces = m_tiles_max * n_tiles;
-    if (args.arrive != nullptr && args.K / 64 >= 2 * kMinPieceStagesIdle) pieces *= kMaxSplit;
-    long long grid = (long long)device_cus();
-    if (pieces < grid) grid = pieces;
-    if (grid < 1) grid = 1;
-    grid = (grid + kXcds - 1) / kXcds * kXcds;   // whole rows of XCDs: the tile order is XCD-aware only then
+    const long long grid = launch_grid(args, 256, SWIGLU, 64, true, device_cus());
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(512), lds, stream, args);
     DMOE_LAUNCH_CHECK("gmm_tile256_fp8_kernel");
     return DMOE_OK;

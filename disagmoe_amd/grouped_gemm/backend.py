@@ -30,6 +30,13 @@ def _sizes_on_device(batch_sizes: torch.Tensor, device: torch.device) -> torch.T
 # hands out a state block (its address is the ``arguments_ptr`` of the reference's
 # API) and the caller allocates the workspace, as experts.py:69-77 does; calls
 # without them use a pair that this module keeps per device and stream.
+#
+# Footprint: a state block is 33 KB; a workspace of the size ``get_arguments``
+# states is 2 x (compute units) x 256 KiB = 128 MiB on a 256-CU device.  Launches
+# that follow each other on one stream can share one workspace (it carries nothing
+# from one launch to the next), so layers should take ``shared_workspace`` rather
+# than allocate one each; only launches that may overlap in time (graphs replayed
+# on different streams) need workspaces of their own.
 
 _STATE_BLOCKS = {}     # address -> the zeroed uint8 tensor behind an arguments_ptr
 _DEFAULTS = {}         # (device index, stream handle) -> (state block, workspace)
@@ -46,17 +53,28 @@ def _new_state_block(device: torch.device) -> torch.Tensor:
     return torch.zeros(_lib.GMM_STATE_BYTES, dtype=torch.uint8, device=device)
 
 
-def _default_state(device: torch.device, stream: int):
-    """``(state block address, workspace address, workspace bytes)`` of stream ``stream`` of
-    ``device``: launches on one stream never overlap, so they can share the pair."""
+def _default_pair(device: torch.device, stream: int):
     key = (device.index, stream)
     pair = _DEFAULTS.get(key)
     if pair is None:
+        if torch.cuda.is_current_stream_capturing():
+            # memory allocated and zero-filled inside a capture belongs to that graph's replays, and the state block
+            # would be shared by every graph recorded on this capture stream
+            raise RuntimeError("a grouped GEMM recorded into a graph needs its own state: pass the arguments_ptr of "
+                               "get_arguments() (and a workspace), as MoEExperts does")
         with torch.cuda.device(device):
             state, ws = _new_state_block(device), torch.empty(workspace_bytes(), dtype=torch.uint8, device=device)
-        pair = (state.data_ptr(), ws.data_ptr(), ws.numel(), state, ws)    # the tensors keep the memory alive
+        pair = (state, ws)
         _DEFAULTS[key] = pair
-    return pair[:3]
+    return pair
+
+
+def shared_workspace(device: torch.device, stream: Optional[int] = None) -> torch.Tensor:
+    """The workspace this module keeps for ``stream`` (default: the current stream) of
+    ``device``: launches on one stream never overlap, so every layer that runs there can
+    use it.  Created on first use, outside any graph capture."""
+    device = torch.device(device)
+    return _default_pair(device, _stream(device) if stream is None else stream)[1]
 
 
 def _state_args(device: torch.device, workspace: Optional[torch.Tensor], arguments_ptr: Optional[int], stream: int):
@@ -66,7 +84,11 @@ def _state_args(device: torch.device, workspace: Optional[torch.Tensor], argumen
 
 def _state_triple(device, workspace, arguments_ptr, stream):
     if arguments_ptr is None and workspace is None:
-        return _default_state(device, stream)
+        if torch.cuda.is_current_stream_capturing():
+            raise RuntimeError("a grouped GEMM recorded into a graph needs its own state: pass the arguments_ptr of "
+                               "get_arguments() (and a workspace), as MoEExperts does")
+        state, ws = _default_pair(device, stream)
+        return state.data_ptr(), ws.data_ptr(), ws.numel()
     if not arguments_ptr:
         raise ValueError("a caller-owned workspace needs the arguments_ptr that get_arguments returned with its size")
     if arguments_ptr not in _STATE_BLOCKS:
@@ -75,6 +97,36 @@ def _state_triple(device, workspace, arguments_ptr, stream):
         return arguments_ptr, None, 0
     assert workspace.dtype == torch.uint8 and workspace.is_contiguous() and workspace.device == device
     return arguments_ptr, workspace.data_ptr(), workspace.numel()
+
+
+def release_arguments(arguments_ptr: int) -> None:
+    """Gives back the state block behind an ``arguments_ptr`` of :func:`get_arguments`
+    (no launch that uses it may be pending or recorded in a live graph)."""
+    _STATE_BLOCKS.pop(arguments_ptr, None)
+
+
+KERNEL_NAMES = {0: "dmoe::gmm_kernel", 1: "dmoe::gmm_direct_kernel", 2: "dmoe::gmm_tile256_kernel",
+                3: "dmoe::gmm_tile256_fp8_kernel"}
+
+
+def launch_plan(rows: int, num_experts: int, K: int, N: int, swiglu: bool = False, fp8: bool = False,
+                workspace_bytes: int = 0, batch_sizes=None) -> dict:
+    """What the library would launch for these shapes (its own answer, dmoe_gmm_plan):
+    kernel, tile rows, wavefronts, workgroups; with ``batch_sizes`` (host values) also the
+    tiles, how many of them are cut along K into how many pieces, and the work items.
+    ``N`` is the number of result columns (``I`` for the swiglu form)."""
+    out = (_lib.ctypes.c_int64 * 9)()
+    sizes = None
+    if batch_sizes is not None:
+        vals = [int(v) for v in (batch_sizes.tolist() if torch.is_tensor(batch_sizes) else batch_sizes)]
+        assert len(vals) == num_experts
+        sizes = (_lib.ctypes.c_int64 * num_experts)(*vals)
+    _lib.call("dmoe_gmm_plan", sizes, int(rows), int(num_experts), int(K), int(N), 1 if swiglu else 0,
+              _lib.FP8_E4M3 if fp8 else _lib.BF16, int(workspace_bytes), out)
+    keys = ("kernel_id", "tile_rows", "wavefronts", "workgroups", "stage_k", "tiles", "cut_tiles", "pieces_per_cut_tile", "items")
+    plan = dict(zip(keys, (int(v) for v in out)))
+    plan["kernel"] = KERNEL_NAMES[plan["kernel_id"]]
+    return plan
 
 
 def _check_operands(a: torch.Tensor, b: torch.Tensor, dtype: torch.dtype) -> torch.device:

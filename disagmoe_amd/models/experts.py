@@ -13,7 +13,41 @@ from ..grouped_gemm import backend as gg
 MAX_BATCH_SIZE = 256  # disagmoe/utils/constants.py:20-22
 
 
-class MoEExperts(torch.nn.Module):
+class _GemmState:
+    """State of a layer's grouped-GEMM launches (experts.py:69-77: ``get_arguments`` and the workspace).
+
+    The 33 KB state block (work counters) is the layer's own: a recorded graph of the layer then shares
+    its scheduler state with no other launch.  The workspace (fp32 partial sums of tiles cut along K,
+    128 MiB on a 256-CU device) carries nothing from one launch to the next, so eager launches use the
+    one the backend keeps for the stream they run on, shared by every layer that runs there.  A layer
+    gets a workspace of its own when one is passed in (``workspace=``; the caller may hand the same
+    tensor to layers whose launches never overlap in time), with ``own_workspace=True``, or when it
+    is recorded into a graph without one (replays may run beside anything; the tensor then comes from
+    the graph's memory pool and stays with the layer)."""
+
+    def _init_gemm_state(self, device, workspace: Optional[torch.Tensor] = None, own_workspace: bool = False):
+        self.workspace_size, self.arguments_ptr = gg.get_arguments(self.num_experts, device)
+        self._gemm_device = torch.device(device)
+        self.workspace = workspace
+        if workspace is None and own_workspace:
+            self.workspace = torch.empty([self.workspace_size], dtype=torch.uint8, device=device)
+
+    def _gemm_state(self) -> dict:
+        ws = self.workspace
+        if ws is None:
+            if torch.cuda.is_current_stream_capturing():
+                ws = self.workspace = torch.empty([self.workspace_size], dtype=torch.uint8, device=self._gemm_device)
+            else:
+                ws = gg.shared_workspace(self._gemm_device)
+        return dict(workspace=ws, arguments_ptr=self.arguments_ptr)
+
+    def __del__(self):
+        ptr = getattr(self, "arguments_ptr", None)
+        if ptr is not None:
+            gg.release_arguments(ptr)
+
+
+class MoEExperts(_GemmState, torch.nn.Module):
     """Fused-w13 SwiGLU experts.
 
     Parameters (experts.py:42-55): ``w13_weight [E, d, 2I]`` (gate = columns
@@ -24,8 +58,10 @@ class MoEExperts(torch.nn.Module):
 
     def __init__(self, hidden_size: int, intermediate_size: int, num_experts: int, tp_size: int = 1,
                  enable_cutlass_cache: bool = True, max_batch_size: int = MAX_BATCH_SIZE,
-                 device: Optional[torch.device] = None, init_std: float = 1.0):
+                 device: Optional[torch.device] = None, init_std: float = 1.0,
+                 workspace: Optional[torch.Tensor] = None, own_workspace: bool = False):
         super().__init__()
+        self._workspace_arg, self._own_workspace_arg = workspace, own_workspace
         self.hidden_size = hidden_size
         self.intermediate_size = intermediate_size
         self.num_experts = num_experts
@@ -58,17 +94,15 @@ class MoEExperts(torch.nn.Module):
         self.cache_up = torch.empty((max_batch_size, self.intermediate_size), dtype=params_dtype, device=dev)
         self.cache_down = torch.empty((max_batch_size, self.hidden_size), dtype=params_dtype, device=dev)
         self.enable_cache = enable_cutlass_cache
-        # state block and workspace of this layer's launches (experts.py:69-77): a captured graph of the layer then
-        # shares its scheduler state with no other launch
-        self.workspace_size, self.arguments_ptr = gg.get_arguments(self.num_experts, dev)
-        self.workspace = torch.empty([self.workspace_size], dtype=torch.uint8, device=dev)
+        # state block of this layer's launches and where their workspace comes from (experts.py:69-77)
+        self._init_gemm_state(dev, getattr(self, "_workspace_arg", None), getattr(self, "_own_workspace_arg", False))
 
     def forward(self, bs: int, hiddens: torch.Tensor, batch_sizes: torch.Tensor) -> torch.Tensor:
         """``gmm(silu(u[:, :I]) * u[:, I:], w2)`` with ``u = gmm(hiddens, w13)``
         (experts.py:92-96); gate-up, SiLU and the product are one kernel.  Below
         ``max_batch_size`` rows the static buffers are used (the reference's
         cached branch, :83-90)."""
-        ws = dict(workspace=getattr(self, "workspace", None), arguments_ptr=getattr(self, "arguments_ptr", None))
+        ws = self._gemm_state()
         if self.enable_cache and bs <= self.gmm_cache_max_batch_size and hiddens.shape[0] <= self.cache_up.shape[0]:
             h = gg.gmm_swiglu(hiddens, self.w13_weight, batch_sizes, c=self.cache_up, **ws)[:hiddens.shape[0]]
             return gg.gmm(h, self.w2_weight, batch_sizes, c=self.cache_down, **ws)[:hiddens.shape[0]]
@@ -78,9 +112,10 @@ class MoEExperts(torch.nn.Module):
     def forward_unfused(self, bs: int, hiddens: torch.Tensor, batch_sizes: torch.Tensor) -> torch.Tensor:
         """The reference's own schedule, statement by statement (experts.py:92-94):
         the gate-up result, SiLU and the product are each rounded to bf16."""
-        up = self.gmm(hiddens, self.w13_weight, batch_sizes)
+        ws = self._gemm_state()
+        up = self.gmm(hiddens, self.w13_weight, batch_sizes, **ws)
         up = self.act_fn(up[:, :self.intermediate_size]) * up[:, self.intermediate_size:]
-        return self.gmm(up, self.w2_weight, batch_sizes)
+        return self.gmm(up, self.w2_weight, batch_sizes, **ws)
 
 
 class MoEExpertsSerial(MoEExperts):
@@ -109,12 +144,13 @@ class MoEExpertsSerial(MoEExperts):
         return torch.cat(results)
 
 
-class MoEExpertsFP8(torch.nn.Module):
+class MoEExpertsFP8(_GemmState, torch.nn.Module):
     """fp8-e4m3 experts (no counterpart in the reference): weights quantised per
     output channel and stored K-contiguous (``w13_q [E, 2I, d]``, ``w2_q [E, d,
     I]``), activations quantised per row on the fly, bf16 in and out."""
 
-    def __init__(self, w13: torch.Tensor, w2: torch.Tensor):
+    def __init__(self, w13: torch.Tensor, w2: torch.Tensor, workspace: Optional[torch.Tensor] = None,
+                 own_workspace: bool = False):
         super().__init__()
         self.num_experts, self.hidden_size, two_i = w13.shape
         self.intermediate_size = two_i // 2
@@ -124,6 +160,7 @@ class MoEExpertsFP8(torch.nn.Module):
         self.w13_scale = torch.nn.Parameter(s13, requires_grad=False)
         self.w2_q = torch.nn.Parameter(q2, requires_grad=False)
         self.w2_scale = torch.nn.Parameter(s2, requires_grad=False)
+        self._init_gemm_state(w13.device, workspace, own_workspace)
 
     def forward(self, bs: int, hiddens: torch.Tensor, batch_sizes: torch.Tensor) -> torch.Tensor:
         xq, xs = gg.quantize_rows(hiddens)
@@ -131,6 +168,7 @@ class MoEExpertsFP8(torch.nn.Module):
 
     def forward_quantized(self, bs: int, xq: torch.Tensor, xs: torch.Tensor, batch_sizes: torch.Tensor) -> torch.Tensor:
         """The same on rows that arrive quantised (``ops.memory.permute_quantize``)."""
-        h = gg.gmm_fp8_swiglu(xq, xs, self.w13_q, self.w13_scale, batch_sizes)
+        ws = self._gemm_state()
+        h = gg.gmm_fp8_swiglu(xq, xs, self.w13_q, self.w13_scale, batch_sizes, **ws)
         hq, hs = gg.quantize_rows(h)
-        return gg.gmm_fp8(hq, hs, self.w2_q, self.w2_scale, batch_sizes)
+        return gg.gmm_fp8(hq, hs, self.w2_q, self.w2_scale, batch_sizes, **ws)

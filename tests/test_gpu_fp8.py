@@ -191,7 +191,8 @@ def test_gmm_fp8_few_stages(variant, K):
     (256, 264, [40, 0, 300]),                          # two k-steps: the prologue's copies are all there are
     (384, 264, [100, 0, 257]),                         # three k-steps: one refill
     (1152, 520, [300, 17, 0, 513, 128]),               # 9 k-steps; a ragged last n-tile
-    (3200, 512, [500, 0, 290]),                        # fewer tiles than compute units, long K: cut along K in uneven pieces
+    (3200, 512, [500, 0, 290]),                        # fewer tiles than compute units
+    (8320, 512, [500, 0, 290]),                        # ... and a long K: cut along K in uneven pieces (65 k-steps)
 ])
 def test_gmm_fp8_tile_of_whole_lines(K, N, sizes, swiglu):
     """The 256-row fp8 tile whose copies fetch whole 128-byte lines (K % 128 == 0; variant 7 picks 256-row tiles)."""
@@ -218,6 +219,94 @@ def test_gmm_fp8_tile_of_whole_lines(K, N, sizes, swiglu):
         assert torch.equal(out, again)                 # pieces are summed in a fixed order
     finally:
         gg.set_tile_variant(0)
+
+
+def _fp8_case(K, N, sizes, swiglu, seed):
+    E, R = len(sizes), sum(sizes)
+    n_w = 2 * N if swiglu else N
+    g = torch.Generator().manual_seed(seed)
+    a = torch.randn(R, K, generator=g).to(torch.bfloat16)
+    w = (torch.randn(E, K, n_w, generator=g) * 0.05).to(torch.bfloat16)
+    bs = torch.tensor(sizes, dtype=torch.int64)
+    aq, a_s = fp8.quantize_rows(a)
+    wq, w_s = fp8.quantize_weight_channels(w)
+    exact = ffn.gmm(fp8.dequantize_rows(aq, a_s, torch.float32), fp8.dequantize_weight(wq, w_s, torch.float32), bs,
+                    out_dtype=torch.float32)
+    if swiglu:
+        exact = torch.nn.functional.silu(exact[:, :N]) * exact[:, N:]
+    return (aq.to(dev()), a_s.to(dev()), wq.to(dev()), w_s.to(dev()), bs.to(dev())), exact
+
+
+@pytest.mark.parametrize("swiglu", [False, True])
+def test_fp8_cut_launches_alternating_operands_on_one_state(swiglu):
+    """Two different problems A, B, A, B, ... through launches of the 256-row fp8 tile that cut their tiles along K, on
+    one state block and one workspace: what a launch leaves there (or a stale copy of it in a cache) belongs to other
+    operands than the next launch's.  Every result against the oracle and against the uncut launch."""
+    announce(test="fp8_split_alternating", swiglu=swiglu)
+    gg.set_tile_variant(7)
+    try:
+        K, N = 8192, 512
+        cases = [_fp8_case(K, N, [500, 0, 290], swiglu, 21), _fp8_case(K, N, [260, 300, 200], swiglu, 22)]
+        run = gg.gmm_fp8_swiglu if swiglu else gg.gmm_fp8
+        size, ptr = gg.get_arguments(3, dev())
+        workspace = torch.empty([size], dtype=torch.uint8, device=dev())
+        for ops, _ in cases:
+            plan = gg.launch_plan(int(ops[4].sum()), 3, K, N, swiglu=swiglu, fp8=True, workspace_bytes=size, batch_sizes=ops[4].cpu())
+            assert plan["kernel_id"] == 3 and plan["pieces_per_cut_tile"] > 1, plan
+        uncut = [run(*ops, arguments_ptr=ptr) for ops, _ in cases]
+        outs = [run(*cases[rep % 2][0], workspace=workspace, arguments_ptr=ptr) for rep in range(6)]
+        torch.cuda.synchronize()
+        for rep, out in enumerate(outs):
+            assert max_rel_err(out, cases[rep % 2][1]) <= 1e-2, (rep, max_rel_err(out, cases[rep % 2][1]))
+            assert max_rel_err(out, uncut[rep % 2].cpu()) <= 2e-2, rep
+            assert torch.equal(out, outs[rep % 2]), rep
+        assert int(gg._STATE_BLOCKS[ptr].count_nonzero()) == 0
+    finally:
+        gg.set_tile_variant(0)
+
+
+def test_two_fp8_graphs_replayed_on_two_streams():
+    """Two fp8 layers, each recorded into a graph of its own on the same capture stream, replayed at the same time on
+    two streams: each layer brings its own state block and workspace, so both give the bits of their serial runs."""
+    announce(test="fp8_two_graphs")
+    E, d, I, R = 4, 1024, 1536, 1800
+    g = torch.Generator().manual_seed(9)
+    layers, inputs, serial, graphs, outs = [], [], [], [], []
+    sizes = [ragged_sizes(E, R, seed=31), ragged_sizes(E, R, seed=32)]
+    for n in range(2):
+        w13 = (torch.randn(E, d, 2 * I, generator=g) * 0.05).to(torch.bfloat16).to(dev())
+        w2 = (torch.randn(E, I, d, generator=g) * 0.05).to(torch.bfloat16).to(dev())
+        layers.append(MoEExpertsFP8(w13, w2))
+        x = torch.randn(R, d, generator=g).to(torch.bfloat16).to(dev())
+        inputs.append((x, sizes[n].to(dev())))
+        serial.append(layers[n].forward(R, *inputs[n]).clone())
+    torch.cuda.synchronize()
+    capture = torch.cuda.Stream()
+    for n in range(2):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=capture):
+            outs.append(layers[n].forward(R, *inputs[n]))
+        graphs.append(graph)
+    assert layers[0].workspace is not None and layers[0].workspace.data_ptr() != layers[1].workspace.data_ptr()
+    assert layers[0].arguments_ptr != layers[1].arguments_ptr
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    for round_ in range(3):
+        for out in outs:
+            out.zero_()
+        torch.cuda.synchronize()
+        for _ in range(4):
+            for n in (1, 0):                           # the graph recorded second goes first
+                with torch.cuda.stream(streams[n]):
+                    graphs[n].replay()
+        torch.cuda.synchronize()
+        for n in range(2):
+            assert torch.equal(outs[n], serial[n]), (round_, n)
+    # a bare call without a state block cannot be recorded
+    with pytest.raises(RuntimeError):
+        with torch.cuda.graph(torch.cuda.CUDAGraph(), stream=capture):
+            xq, xs = gg.quantize_rows(inputs[0][0])
+            gg.gmm_fp8_swiglu(xq, xs, layers[0].w13_q, layers[0].w13_scale, inputs[0][1])
+    torch.cuda.synchronize()
 
 
 @pytest.mark.parametrize("swiglu", [False, True])

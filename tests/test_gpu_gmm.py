@@ -247,33 +247,12 @@ def _split_case(E, R, K, N, seed, swiglu, trans_b):
     return a.to(dev()), b.to(dev()), sizes.to(dev()), ref
 
 
-def _expected_split(sizes, tile_rows, n_out, swiglu, K, workspace_bytes):
-    """The launch's plan (csrc/gmm_common.h plan_work, csrc/gmm_direct.h launch_direct_one, csrc/gmm_tile256.h launch_tile256_one) restated: pieces per tile
-    of the last round, 1 if nothing is cut."""
-    cus = torch.cuda.get_device_properties(0).multi_processor_count
-    n_tiles = -(-n_out // (128 if swiglu else 256))
-    rows, E = int(sum(sizes)), len(sizes)
-    pieces = (rows // tile_rows + E) * n_tiles
-    if K // 32 >= 2 * 24:
-        pieces *= 8                                  # a launch that may cut tiles may use more workgroups than it has tiles
-    grid = -(-max(min(cus, pieces), 1) // 8) * 8
-    tiles = sum(-(-n // tile_rows) for n in sizes) * n_tiles
-    stages, rem = K // 32, tiles % grid
-    max_pieces = workspace_bytes // (tile_rows * 256 * 4)
-    if rem == 0 or rem > 8192 // (8 if tile_rows == 256 else 4):
-        return 1
-    if tiles // grid > 3:
-        return 1
-    best, best_cost = 1, stages + 8
-    min_piece = 24 if tiles < grid else 88           # pieces may be short where they run on compute units that have no tile
-    for p in range(2, 9):
-        if rem * p > max_pieces or stages // p < min_piece:
-            break
-        rounds = -(-rem * p // grid)
-        cost = rounds * (-(-stages // p) + 20) + 4 + 4 * p
-        if cost < best_cost:
-            best, best_cost = p, cost
-    return 1 if best == 1 or best_cost * 100 > (85 if stages // best < 88 else 92) * (stages + 8) else best
+def _expected_split(sizes, n_out, swiglu, K, workspace_bytes, fp8=False):
+    """Pieces per tile of the last round (1: nothing is cut) and the tile rows, as the library itself plans the launch
+    (dmoe_gmm_plan, which runs the code the launch runs)."""
+    plan = gg.launch_plan(int(sum(sizes)), len(sizes), K, n_out, swiglu=swiglu, fp8=fp8, workspace_bytes=workspace_bytes,
+                          batch_sizes=sizes)
+    return plan["pieces_per_cut_tile"], plan["tile_rows"]
 
 
 @pytest.mark.parametrize("variant", [5, 6, 7, 0])
@@ -297,15 +276,47 @@ def test_gmm_tail_tiles_cut_along_k(variant, swiglu, trans_b, E, R, K, N):
     assert torch.equal(fn(a, b, sizes, trans_b=trans_b), outs[0])
     # pieces were written where the plan cuts tiles (the head of the workspace no longer holds the fill pattern), and
     # only there; the cases are chosen so that every forced tile height cuts at least once
-    tile_rows = {5: 64, 6: 128, 7: 256}.get(variant)
-    if tile_rows is not None:
-        split = _expected_split(sizes.cpu().tolist(), tile_rows, N, swiglu, K, size)
-        print(f"[split] tile rows {tile_rows}: {split} pieces per tile of the last round")
-        assert bool((workspace[:4096] == 0xA5).all()) == (split == 1)
+    split, tile_rows = _expected_split(sizes.cpu().tolist(), N, swiglu, K, size)
+    print(f"[split] tile rows {tile_rows}: {split} pieces per tile of the last round")
+    assert variant not in (5, 6, 7) or tile_rows == {5: 64, 6: 128, 7: 256}[variant]
+    assert bool((workspace[:4096] == 0xA5).all()) == (split == 1)
     # without a workspace nothing is cut: the same product summed in one piece
     whole = fn(a, b, sizes, trans_b=trans_b, arguments_ptr=ptr)
     assert max_rel_err(whole, ref) <= TOL_BF16
     assert max_rel_err(whole, outs[0].cpu()) <= 2e-2
+
+
+@pytest.mark.parametrize("variant", [5, 6, 7])
+@pytest.mark.parametrize("swiglu", [False, True])
+def test_cut_launches_alternating_operands_on_one_state(variant, swiglu):
+    # Two different problems A, B, A, B, ... through cut launches that share one state block and one workspace: a
+    # partial sum or an arrival count left over from the launch before (or a stale copy of it in some cache) would
+    # show, because the launch before had other operands.  Every result against the oracle and against the same
+    # launch without a workspace (nothing cut).
+    announce(test="gmm_split_alternating", variant=variant, swiglu=swiglu)
+    gg.set_tile_variant(variant)
+    E, K, N = 3, 8192, 512
+    cases = [_split_case(E, 700, K, N, seed=11, swiglu=swiglu, trans_b=False),
+             _split_case(E, 640, K, N, seed=12, swiglu=swiglu, trans_b=False)]
+    fn = gg.gmm_swiglu if swiglu else gg.gmm
+    size, ptr = gg.get_arguments(E, dev())
+    workspace = torch.empty([size], dtype=torch.uint8, device=dev())
+    for a, b, sizes, _ in cases:
+        split, _rows = _expected_split(sizes.cpu().tolist(), N, swiglu, K, size)
+        assert split > 1
+    uncut = [fn(a, b, sizes, arguments_ptr=ptr) for a, b, sizes, _ in cases]
+    outs = []
+    for rep in range(6):
+        a, b, sizes, _ = cases[rep % 2]
+        outs.append(fn(a, b, sizes, workspace=workspace, arguments_ptr=ptr))     # back to back, no synchronisation
+    torch.cuda.synchronize()
+    for rep, out in enumerate(outs):
+        ref = cases[rep % 2][3]
+        assert max_rel_err(out, ref) <= TOL_BF16, (rep, max_rel_err(out, ref))
+        assert max_rel_err(out, uncut[rep % 2].cpu()) <= 2e-2, rep
+        assert torch.equal(out, outs[rep % 2]), rep
+    assert int(gg._STATE_BLOCKS[ptr].count_nonzero()) == 0
+    gg.set_tile_variant(0)
 
 
 def test_gmm_launches_on_two_streams_keep_their_own_state():

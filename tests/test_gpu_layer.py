@@ -28,6 +28,7 @@ def _layer_from(w13, w2):
     layer.gmm_cache_max_batch_size = 0
     from disagmoe_amd.grouped_gemm import backend as gg
     layer.gmm = gg.gmm
+    layer._init_gemm_state(w13.device)
     return layer
 
 

@@ -51,6 +51,36 @@ def test_noalloc_route_matches_route_on_consecutive_calls():
             assert got[0].cpu().tolist() == m_ref and got[1].cpu().tolist() == cnt_ref
 
 
+def test_noalloc_route_recorded_into_a_graph():
+    """The caller the entry point is for: recorded once into a graph (after a first eager call, which looks up the
+    built-in buffer's address), replayed with new ids after eager calls of other sizes have used the same buffer."""
+    from oracle import routing
+    R, E = 20000, 16                                                  # 40 chunks: the histograms go through the buffer
+    g = torch.Generator().manual_seed(5)
+    ids = torch.randint(0, E, (R,), generator=g, dtype=torch.int32).to(dev())
+    mappings = torch.full((R,), -7, dtype=torch.int64, device=dev())
+    batch_sizes = torch.full((E,), -7, dtype=torch.int64, device=dev())
+    offsets = torch.full((E + 1,), -7, dtype=torch.int64, device=dev())
+    _route(ids, E, _lib.ORDER_REFERENCE, noalloc=True)
+    announce(test="route_noalloc_graph", R=R, E=E)
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        _lib.call("dmoe_route_noalloc", ids.data_ptr(), _lib.I32, R, E, _lib.ORDER_REFERENCE, mappings.data_ptr(), _lib.I64,
+                  batch_sizes.data_ptr(), offsets.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    for rep in range(3):
+        new_ids = torch.randint(0, E, (R,), generator=g, dtype=torch.int32)
+        new_ids[new_ids == 3] = 4
+        ids.copy_(new_ids)
+        other = torch.randint(0, 64, (49152 if rep % 2 == 0 else 9000,), generator=g, dtype=torch.int32).to(dev())
+        _route(other, 64, _lib.ORDER_STABLE, noalloc=True)            # an eager call of another size in between
+        graph.replay()
+        torch.cuda.synchronize()
+        m_ref, cnt_ref = routing.get_mappings_from_exp_ids(new_ids, E)
+        assert mappings.cpu().tolist() == m_ref and batch_sizes.cpu().tolist() == cnt_ref, rep
+        assert offsets.cpu().tolist() == [0] + torch.tensor(cnt_ref).cumsum(0).tolist()
+
+
 def test_noalloc_route_refuses_what_does_not_fit():
     limit = ctypes.c_size_t(0)
     _lib.call("dmoe_route_noalloc_max_bytes", ctypes.byref(limit))

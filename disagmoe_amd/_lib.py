@@ -58,7 +58,7 @@ SIGNATURES = {
 #: exported for the library's own tests and benchmarks, not declared in include/dmoe.h (csrc/tuning.h)
 TEST_HOOKS = {
     "dmoe_gmm_tune": (c_int, [c_int]),
-    "dmoe_gmm_plan": (c_int, [c_void_p, c_int64, c_int, c_int64, c_int64, c_int, c_int, c_size_t, c_void_p]),
+    "dmoe_gmm_plan": (c_int, [c_void_p, c_int64, c_int, c_int64, c_int64, c_int, c_int, c_int, c_size_t, c_void_p]),
 }
 GMM_STATE_BYTES = 33024
 

@@ -473,7 +473,7 @@ static int bind_state(GmmArgs &args, void *state, void *workspace, size_t worksp
 
 // Kernel, tile rows and grid of a launch, from what the host knows (the shapes, not how the rows split over the experts).
 // The one place where that is decided: launch_by_rows dispatches on the result and dmoe_gmm_plan reports it.
-static GmmLaunch choose_launch(const GmmArgs &args, bool swiglu, bool fp8) {
+static GmmLaunch choose_launch(const GmmArgs &args, bool trans_b, bool swiglu, bool fp8) {
     const int cus = device_cus();
     GmmLaunch L{};
     if (g_variant >= 1 && g_variant <= 4) {   // test hook: the register-staged kernel with a fixed tile
@@ -502,7 +502,7 @@ static GmmLaunch choose_launch(const GmmArgs &args, bool swiglu, bool fp8) {
             tile_rows = avg <= 64 ? 64 : (avg <= 160 ? 128 : 256);
             while (tile_rows > 64 && (args.rows / tile_rows + (args.E + 1) / 2) * n_tiles * 2 < cus) tile_rows /= 2;
         }
-        if (g_variant >= 5) tile_rows = g_variant == 5 ? 64 : (g_variant == 6 ? 128 : 256);   // test hook: fixed tile rows
+        if (g_variant >= 5) tile_rows = g_variant == 5 ? 64 : (g_variant == 6 ? 128 : 256);   // test hook: fixed tile rows (7, 8: 256)
         L.tile_rows = tile_rows;
         // global -> LDS kernels: whole stages (32 k of bf16, 64 of fp8), 32-bit offsets inside one expert's weights
         const bool direct = fp8 ? (args.K % 64 == 0 && (long long)args.K * args.N < (1ll << 32))
@@ -510,6 +510,8 @@ static GmmLaunch choose_launch(const GmmArgs &args, bool swiglu, bool fp8) {
         if (!direct) {
             L.kernel = kKernelStaged;
             L.waves = tile_rows == 256 ? 8 : 4;
+        } else if (tile_rows == 256 && !fp8 && !trans_b && g_variant == 8) {
+            L.kernel = kKernelWave128; L.waves = 4;
         } else if (tile_rows == 256 && !fp8) {
             L.kernel = kKernelTile256; L.waves = 8;
         } else if (tile_rows == 256 && args.K % 128 == 0) {
@@ -528,13 +530,14 @@ static GmmLaunch choose_launch(const GmmArgs &args, bool swiglu, bool fp8) {
 
 template <bool TRANS_B, bool SWIGLU, bool FP8>
 static int launch_by_rows(const GmmArgs &args, hipStream_t stream) {
-    const GmmLaunch L = choose_launch(args, SWIGLU, FP8);
+    const GmmLaunch L = choose_launch(args, TRANS_B, SWIGLU, FP8);
     if (L.kernel == kKernelStaged) {
         if (L.tile_rows == 64) return launch_one<64, 256, 1, 4, TRANS_B, SWIGLU, FP8>(args, stream);
         if (L.tile_rows == 128) return launch_one<128, 256, 1, 4, TRANS_B, SWIGLU, FP8>(args, stream);
         if (L.waves == 4) return launch_one<256, 256, 2, 2, TRANS_B, SWIGLU, FP8>(args, stream);
         return launch_one<256, 256, 2, 4, TRANS_B, SWIGLU, FP8>(args, stream);
     }
+    if (L.kernel == kKernelWave128) return launch_wave128(args, SWIGLU, stream);
     if constexpr (FP8) return launch_direct_fp8(args, L.tile_rows, SWIGLU, stream);
     else return launch_direct_bf16(args, L.tile_rows, TRANS_B, SWIGLU, stream);
 }
@@ -563,7 +566,7 @@ static int check_gmm(const char *who, const void *a, const void *b, const void *
 using namespace dmoe;
 
 extern "C" int dmoe_gmm_tune(int variant) {
-    DMOE_REQUIRE(variant >= 0 && variant <= 7, DMOE_ERR_ARG, "dmoe_gmm_tune: variant %d outside [0, 7]", variant);
+    DMOE_REQUIRE(variant >= 0 && variant <= 8, DMOE_ERR_ARG, "dmoe_gmm_tune: variant %d outside [0, 8]", variant);
     g_variant = variant;
     return DMOE_OK;
 }
@@ -571,8 +574,8 @@ extern "C" int dmoe_gmm_tune(int variant) {
 // What a launch with these shapes would run (see tuning.h).  out: [0] kernel (GmmKernelId), [1] tile rows, [2] wavefronts
 // per workgroup, [3] workgroups, [4] k per stage unit; and, when the sizes are given (host memory), what the kernel
 // derives from them on the device: [5] tiles, [6] tiles cut along K, [7] pieces per cut tile, [8] work items; -1 without.
-extern "C" int dmoe_gmm_plan(const int64_t *host_batch_sizes, int64_t rows, int E, int64_t K, int64_t N, int swiglu,
-                             int dtype, size_t workspace_bytes, int64_t *out) {
+extern "C" int dmoe_gmm_plan(const int64_t *host_batch_sizes, int64_t rows, int E, int64_t K, int64_t N, int trans_b,
+                             int swiglu, int dtype, size_t workspace_bytes, int64_t *out) {
     DMOE_REQUIRE(out != nullptr, DMOE_ERR_ARG, "dmoe_gmm_plan: null output");
     DMOE_REQUIRE(dtype == DMOE_BF16 || dtype == DMOE_FP8_E4M3, DMOE_ERR_DTYPE, "dmoe_gmm_plan: dtype %d", dtype);
     const bool fp8 = dtype == DMOE_FP8_E4M3;
@@ -582,7 +585,7 @@ extern "C" int dmoe_gmm_plan(const int64_t *host_batch_sizes, int64_t rows, int 
     GmmArgs args{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, rows, E, (int)K, (int)n_cols, (int)N};
     args.arrive = workspace_bytes > 0 ? (unsigned int *)out : nullptr;   // only tested against nullptr
     args.partial_bytes = (long long)workspace_bytes;
-    const GmmLaunch L = choose_launch(args, swiglu != 0, fp8);
+    const GmmLaunch L = choose_launch(args, trans_b != 0 || fp8, swiglu != 0, fp8);
     out[0] = L.kernel; out[1] = L.tile_rows; out[2] = L.waves; out[3] = L.grid; out[4] = L.stage_k;
     out[5] = out[6] = out[7] = out[8] = -1;
     if (host_batch_sizes != nullptr) {

@@ -10,6 +10,7 @@ namespace dmoe {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef int i32x8 __attribute__((ext_vector_type(8)));
 
@@ -317,7 +318,7 @@ __device__ __forceinline__ bool meet_pieces(AccT (&acc)[FM][FN], const GmmArgs &
 }
 
 // ---- the launch a problem gets (host) -------------------------------------------------------------------
-enum GmmKernelId { kKernelStaged = 0, kKernelDirect = 1, kKernelTile256 = 2, kKernelTile256Fp8 = 3 };
+enum GmmKernelId { kKernelStaged = 0, kKernelDirect = 1, kKernelTile256 = 2, kKernelTile256Fp8 = 3, kKernelWave128 = 4 };
 struct GmmLaunch {
     int kernel;        // GmmKernelId
     int tile_rows;     // rows of a tile (64, 128, 256); a tile has 256 columns of b
@@ -344,5 +345,6 @@ inline long long launch_grid(const GmmArgs &args, int tile_rows, bool swiglu, in
 int launch_direct_bf16(const GmmArgs &args, int tile_rows, bool trans_b, bool swiglu, hipStream_t stream);
 int launch_direct_fp8(const GmmArgs &args, int tile_rows, bool swiglu, hipStream_t stream);
 int launch_tile256_fp8(const GmmArgs &args, bool swiglu, hipStream_t stream);
+int launch_wave128(const GmmArgs &args, bool swiglu, hipStream_t stream);
 
 }  // namespace dmoe

@@ -26,8 +26,6 @@
 
 namespace dmoe {
 
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-
 template <bool TRANS_B, bool SWIGLU>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void gmm_tile256_kernel(const GmmArgs p) {

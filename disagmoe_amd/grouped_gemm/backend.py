@@ -106,11 +106,11 @@ def release_arguments(arguments_ptr: int) -> None:
 
 
 KERNEL_NAMES = {0: "dmoe::gmm_kernel", 1: "dmoe::gmm_direct_kernel", 2: "dmoe::gmm_tile256_kernel",
-                3: "dmoe::gmm_tile256_fp8_kernel"}
+                3: "dmoe::gmm_tile256_fp8_kernel", 4: "dmoe::gmm_wave128_kernel"}
 
 
 def launch_plan(rows: int, num_experts: int, K: int, N: int, swiglu: bool = False, fp8: bool = False,
-                workspace_bytes: int = 0, batch_sizes=None) -> dict:
+                workspace_bytes: int = 0, batch_sizes=None, trans_b: bool = False) -> dict:
     """What the library would launch for these shapes (its own answer, dmoe_gmm_plan):
     kernel, tile rows, wavefronts, workgroups; with ``batch_sizes`` (host values) also the
     tiles, how many of them are cut along K into how many pieces, and the work items.
@@ -121,7 +121,7 @@ def launch_plan(rows: int, num_experts: int, K: int, N: int, swiglu: bool = Fals
         vals = [int(v) for v in (batch_sizes.tolist() if torch.is_tensor(batch_sizes) else batch_sizes)]
         assert len(vals) == num_experts
         sizes = (_lib.ctypes.c_int64 * num_experts)(*vals)
-    _lib.call("dmoe_gmm_plan", sizes, int(rows), int(num_experts), int(K), int(N), 1 if swiglu else 0,
+    _lib.call("dmoe_gmm_plan", sizes, int(rows), int(num_experts), int(K), int(N), 1 if trans_b else 0, 1 if swiglu else 0,
               _lib.FP8_E4M3 if fp8 else _lib.BF16, int(workspace_bytes), out)
     keys = ("kernel_id", "tile_rows", "wavefronts", "workgroups", "stage_k", "tiles", "cut_tiles", "pieces_per_cut_tile", "items")
     plan = dict(zip(keys, (int(v) for v in out)))

@@ -43,7 +43,7 @@ def test_reference_gemm_case():
     assert max_rel_err(y, ffn.gmm(x.cpu(), w1.cpu(), batch_sizes)) <= TOL_BF16
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, 8])
 @pytest.mark.parametrize("E,R,K,N", [(1, 300, 256, 256), (4, 1000, 128, 512), (8, 777, 320, 264), (3, 64, 72, 40),
                                      (5, 1500, 512, 768)])
 @pytest.mark.parametrize("trans_b", [False, True])
@@ -85,7 +85,7 @@ def test_gmm_single_expert_equals_matmul_and_zero_sizes():
     assert (guard[513:] == 5.0).all()
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, 8])
 @pytest.mark.parametrize("trans_b", [False, True])
 def test_gmm_swiglu(variant, trans_b):
     announce(test="gmm_swiglu", variant=variant, trans_b=trans_b)
@@ -212,7 +212,7 @@ def test_gmm_decode_sized_batch_on_tall_tiles(trans_b, K):
     assert max_rel_err(h, ref_h) <= TOL_BF16
 
 
-@pytest.mark.parametrize("variant", [0, 5, 6, 7])
+@pytest.mark.parametrize("variant", [0, 5, 6, 7, 8])
 @pytest.mark.parametrize("K", [32, 64, 96])
 def test_gmm_few_stages(variant, K):
     # one, two and three 32-k stages: fewer than the LDS pipeline is deep (its prologue, tail and the staging of the
@@ -255,7 +255,7 @@ def _expected_split(sizes, n_out, swiglu, K, workspace_bytes, fp8=False):
     return plan["pieces_per_cut_tile"], plan["tile_rows"]
 
 
-@pytest.mark.parametrize("variant", [5, 6, 7, 0])
+@pytest.mark.parametrize("variant", [5, 6, 7, 8, 0])
 @pytest.mark.parametrize("swiglu,trans_b", [(False, False), (True, False), (False, True), (True, True)])
 @pytest.mark.parametrize("E,R,K,N", [(2, 200, 8192, 256), (3, 700, 8192, 512), (2, 150, 16384, 256), (8, 1500, 1024, 768)])
 def test_gmm_tail_tiles_cut_along_k(variant, swiglu, trans_b, E, R, K, N):
@@ -278,7 +278,7 @@ def test_gmm_tail_tiles_cut_along_k(variant, swiglu, trans_b, E, R, K, N):
     # only there; the cases are chosen so that every forced tile height cuts at least once
     split, tile_rows = _expected_split(sizes.cpu().tolist(), N, swiglu, K, size)
     print(f"[split] tile rows {tile_rows}: {split} pieces per tile of the last round")
-    assert variant not in (5, 6, 7) or tile_rows == {5: 64, 6: 128, 7: 256}[variant]
+    assert variant not in (5, 6, 7, 8) or tile_rows == {5: 64, 6: 128, 7: 256, 8: 256}[variant]
     assert bool((workspace[:4096] == 0xA5).all()) == (split == 1)
     # without a workspace nothing is cut: the same product summed in one piece
     whole = fn(a, b, sizes, trans_b=trans_b, arguments_ptr=ptr)
@@ -286,7 +286,7 @@ def test_gmm_tail_tiles_cut_along_k(variant, swiglu, trans_b, E, R, K, N):
     assert max_rel_err(whole, outs[0].cpu()) <= 2e-2
 
 
-@pytest.mark.parametrize("variant", [5, 6, 7])
+@pytest.mark.parametrize("variant", [5, 6, 7, 8])
 @pytest.mark.parametrize("swiglu", [False, True])
 def test_cut_launches_alternating_operands_on_one_state(variant, swiglu):
     # Two different problems A, B, A, B, ... through cut launches that share one state block and one workspace: a

@@ -510,7 +510,7 @@ static GmmLaunch choose_launch(const GmmArgs &args, bool trans_b, bool swiglu, b
         if (!direct) {
             L.kernel = kKernelStaged;
             L.waves = tile_rows == 256 ? 8 : 4;
-        } else if (tile_rows == 256 && !fp8 && !trans_b && g_variant == 8) {
+        } else if (tile_rows == 256 && !fp8 && !trans_b && args.K >= 256 && args.K % 128 == 0 && g_variant == 8) {
             L.kernel = kKernelWave128; L.waves = 4;
         } else if (tile_rows == 256 && !fp8) {
             L.kernel = kKernelTile256; L.waves = 8;

@@ -236,7 +236,8 @@ struct WorkItem {
     int piece;
     int split_tile;
 };
-template <int BM>
+// kAlign: the pieces of a split tile begin at multiples of kAlign stages (`stages` is one).
+template <int BM, int kAlign = 1>
 __device__ __forceinline__ WorkItem decode_item(long long q, int G, const WorkPlan &w, int stages, int n_tiles, int E,
                                                 const int *s_tile_start, const int *s_row_start) {
     const long long L = item_order(q, G, w.items);
@@ -248,8 +249,8 @@ __device__ __forceinline__ WorkItem decode_item(long long q, int G, const WorkPl
         it.piece = (int)(r / w.rem);
         it.split_tile = (int)(r - (long long)it.piece * w.rem);
         tile = w.whole + it.split_tile;
-        it.s_lo = (int)((long long)stages * it.piece / w.split);
-        it.s_cnt = (int)((long long)stages * (it.piece + 1) / w.split) - it.s_lo;
+        it.s_lo = (int)((long long)stages * it.piece / w.split) / kAlign * kAlign;
+        it.s_cnt = (int)((long long)stages * (it.piece + 1) / w.split) / kAlign * kAlign - it.s_lo;
     }
     it.tile = decode_tile<BM>(tile, n_tiles, E, s_tile_start, s_row_start);
     return it;

@@ -55,7 +55,7 @@ def test_host_side_argument_errors():
     header = open(os.path.join(ROOT, "include", "dmoe.h")).read()
     assert f"#define DMOE_GMM_STATE_BYTES {_lib.GMM_STATE_BYTES}" in header
     assert "dmoe_gmm_tune" not in header and hasattr(lib, "dmoe_gmm_tune")      # a test hook, not public ABI
-    assert lib.dmoe_gmm_tune(8) == -1 and lib.dmoe_gmm_tune(4) == 0 and lib.dmoe_gmm_tune(0) == 0
+    assert lib.dmoe_gmm_tune(9) == -1 and lib.dmoe_gmm_tune(4) == 0 and lib.dmoe_gmm_tune(0) == 0
     with pytest.raises(_lib.DmoeError):
         _lib.call("dmoe_gmm_tune", -1)
     # empty problems succeed without touching the device

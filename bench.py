@@ -143,12 +143,20 @@ def main() -> int:
         layer._gemm_state = lambda: gemm_state
     torch.cuda.synchronize()
 
+    # bf16: where the batch is small enough for it to pay, the gate-up kernel fetches the tokens' rows by their place in
+    # the expert-sorted order and no permute kernel runs (the same result bit for bit)
+    fetch_rows = (not w.fp8) and (not args.no_split) and layer.takes_rows(w.T, w.R)
+
     def step():
-        mappings, batch_sizes, _ = memory.route_tokens(ids, w.E)
         if w.fp8:   # the routed rows are quantised on their way into the expert-sorted buffer
+            mappings, batch_sizes, _ = memory.route_tokens(ids, w.E)
             xq, xs = memory.permute_quantize(x, mappings)
             y = layer.forward_quantized(w.R, xq, xs, batch_sizes)
+        elif fetch_rows:
+            mappings, batch_sizes, _, row_token = memory.route_tokens_with_sources(ids, w.E)
+            y = layer.forward_rows(x, row_token, batch_sizes)
         else:
+            mappings, batch_sizes, _ = memory.route_tokens(ids, w.E)
             permuted = memory.permute_tokens_cuda(x, mappings)
             y = layer.forward(w.R, permuted, batch_sizes)
         return memory.combine_tokens(y, mappings, gates)
@@ -346,6 +354,8 @@ def main() -> int:
         "vs_baseline": None, "dtype": "fp8_e4m3" if w.fp8 else "bf16", "data": "synthetic",
         "config": {"workload": w.name, "E": w.E, "d": w.d, "ffn": w.I, "T": w.T, "top_k": w.k,
                    "routed_rows": w.R, "routing": w.routing, "tile_variant": args.variant,
+                   "permute": ("fetched by the gate-up kernel (dmoe_gmm_swiglu_rows): no permute launch in the timed step"
+                               if fetch_rows else "fused with the row quantiser" if w.fp8 else "its own kernel"),
                    "tail_tiles_cut_along_k": not args.no_split},
         "roofline": roofline,
         "stage_timing": "ms = per launch with several launches inside one HIP event pair on the launch stream (5 for the "

@@ -24,6 +24,8 @@ SIGNATURES = {
     "dmoe_route_scratch_bytes": (c_int, [c_int64, c_int, POINTER(c_size_t)]),
     "dmoe_route": (c_int, [c_void_p, c_int, c_int64, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p,
                            c_void_p, c_size_t, c_void_p]),
+    "dmoe_route_sources": (c_int, [c_void_p, c_int, c_int64, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int,
+                                   c_void_p, c_void_p, c_size_t, c_void_p]),
     "dmoe_route_noalloc_max_bytes": (c_int, [POINTER(c_size_t)]),
     "dmoe_route_noalloc": (c_int, [c_void_p, c_int, c_int64, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p,
                                    c_void_p]),
@@ -45,6 +47,8 @@ SIGNATURES = {
                          c_void_p, c_void_p, c_size_t, c_void_p]),
     "dmoe_gmm_swiglu": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int64, c_int64, c_int,
                                 c_int, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "dmoe_gmm_swiglu_rows": (c_int, [c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int64,
+                                     c_int64, c_int, c_void_p, c_void_p, c_size_t, c_void_p]),
     "dmoe_gmm_workspace_bytes": (c_int, [c_int, POINTER(c_size_t)]),
     "dmoe_quant_rows": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int, c_void_p]),
     "dmoe_permute_quant": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int,

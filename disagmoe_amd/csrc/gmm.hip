@@ -459,6 +459,7 @@ static int own_slot(hipStream_t stream, SchedSlot **out) {
 
 static int bind_state(GmmArgs &args, void *state, void *workspace, size_t workspace_bytes, hipStream_t stream) {
     args.arrive = nullptr; args.partials = nullptr; args.partial_bytes = 0;
+    args.a_rows = nullptr; args.a_src_rows = 0;
     if (state == nullptr) return own_slot(stream, &args.sched);
     DMOE_REQUIRE(((uintptr_t)state & 255) == 0, DMOE_ERR_WORKSPACE, "grouped GEMM: the state block must be 256-byte aligned");
     args.sched = (SchedSlot *)state;
@@ -646,6 +647,26 @@ extern "C" int dmoe_gmm_swiglu(const void *a, const void *b, void *h, const int6
     if (rc != DMOE_OK) return rc;
     return trans_b ? launch_by_rows<true, true, false>(args, (hipStream_t)stream)
                    : launch_by_rows<false, true, false>(args, (hipStream_t)stream);
+}
+
+extern "C" int dmoe_gmm_swiglu_rows(const void *x, const int32_t *row_token, int64_t T, const void *b, void *h,
+                                    const int64_t *batch_sizes, int64_t rows, int E, int64_t K, int64_t I, int dtype,
+                                    void *state, void *workspace, size_t workspace_bytes, void *stream) {
+    DMOE_REQUIRE(dtype == DMOE_BF16, DMOE_ERR_DTYPE, "dmoe_gmm_swiglu_rows: dtype %d (bf16 only)", dtype);
+    int rc = check_gmm("dmoe_gmm_swiglu_rows", x, b, h, batch_sizes, rows, E, K, I, 32);
+    if (rc != DMOE_OK) return rc;
+    DMOE_REQUIRE(T > 0 && T * K * 2 < (1ll << 32), DMOE_ERR_SHAPE,
+                 "dmoe_gmm_swiglu_rows: T=%lld rows of K=%lld must be fewer than 4 GiB", (long long)T, (long long)K);
+    DMOE_REQUIRE(K * 2 * I * 2 < (1ll << 32), DMOE_ERR_SHAPE,
+                 "dmoe_gmm_swiglu_rows: one expert's weights (K=%lld x 2I=%lld) must be fewer than 4 GiB", (long long)K, (long long)(2 * I));
+    DMOE_REQUIRE(rows == 0 || row_token != nullptr, DMOE_ERR_ARG, "dmoe_gmm_swiglu_rows: null row_token");
+    if (rows == 0) return DMOE_OK;
+    GmmArgs args{(const char *)x, (const char *)b, (char *)h, batch_sizes, nullptr, nullptr, rows, E, (int)K, (int)(2 * I), (int)I};
+    rc = bind_state(args, state, workspace, workspace_bytes, (hipStream_t)stream);
+    if (rc != DMOE_OK) return rc;
+    args.a_rows = row_token;
+    args.a_src_rows = T;
+    return launch_tile256_rows(args, (hipStream_t)stream);
 }
 
 extern "C" int dmoe_gmm_fp8(const void *a, const float *a_scale, const void *b, const float *b_scale, void *c,

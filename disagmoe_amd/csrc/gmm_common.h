@@ -34,6 +34,9 @@ struct GmmArgs {
     unsigned int *arrive;         // arrival counters of the split tiles, zero between launches (nullptr: no splitting)
     float *partials;              // fp32 partial results of the pieces of split tiles
     long long partial_bytes;      // capacity of `partials`
+    // (gmm_tile256_kernel's gathering form) row r of the product is row a_rows[r] of `a`, which has a_src_rows rows
+    const int32_t *a_rows;
+    long long a_src_rows;
 };
 
 // ---- work distribution ---------------------------------------------------------------------------
@@ -347,5 +350,6 @@ int launch_direct_bf16(const GmmArgs &args, int tile_rows, bool trans_b, bool sw
 int launch_direct_fp8(const GmmArgs &args, int tile_rows, bool swiglu, hipStream_t stream);
 int launch_tile256_fp8(const GmmArgs &args, bool swiglu, hipStream_t stream);
 int launch_wave128(const GmmArgs &args, bool swiglu, hipStream_t stream);
+int launch_tile256_rows(const GmmArgs &args, hipStream_t stream);
 
 }  // namespace dmoe

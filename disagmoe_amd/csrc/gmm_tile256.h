@@ -26,7 +26,11 @@
 
 namespace dmoe {
 
-template <bool TRANS_B, bool SWIGLU>
+// GATHER: row r of the product is row p.a_rows[r] of a (the tokens, in their own order): the permute that sorts the
+// routed rows by expert needs no launch and no copy of the rows.  A tile's row numbers are fetched and waited for before
+// the epilogue of the tile before it, when nothing else of the wavefront is in flight: behind the epilogue the same
+// wait would also be one for the epilogue's stores.
+template <bool TRANS_B, bool SWIGLU, bool GATHER = false>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void gmm_tile256_kernel(const GmmArgs p) {
     constexpr int kDM = 256, NW = 8, WN = 4;
@@ -108,6 +112,7 @@ void gmm_tile256_kernel(const GmmArgs p) {
     int part = -1, split_tile = 0;
     uint64_t a_base = 0, b_exp = 0;
     uint32_t a_off[CA], b_off[CB];
+    int a_tok[GATHER ? CA : 1];                            // GATHER: source rows of this lane's A rows
     // the expert of the item has a single m-tile: its weights pass through this workgroup once and through no other, so
     // their copies take the non-temporal policy (wave-uniform)
     bool b_once = false;
@@ -117,20 +122,32 @@ void gmm_tile256_kernel(const GmmArgs p) {
         const int base = (SWIGLU && slot >= kDN / 2) ? n_out + n0 : n0;
         return base + (rh < n_out - n0 ? rh : 0);          // slots past the end read a valid column (never stored)
     };
-    auto open_tile = [&](long long q) {
-        const WorkItem it = decode_item<kDM>(q, G, plan, S_all, n_tiles, E, s_tile_start, s_row_start);
+    auto locate = [&](long long q) { return decode_item<kDM>(q, G, plan, S_all, n_tiles, E, s_tile_start, s_row_start); };
+    // GATHER: asks for the row numbers of this lane's A rows of item `it`
+    auto fetch_rows = [&](const WorkItem &it) {
+        if constexpr (GATHER) {
+#pragma unroll
+            for (int i = 0; i < CA; ++i) {
+                int r = (i * NW + wave) * 16 + kc_row;
+                if (r >= it.tile.rows_e) r = it.tile.rows_e - 1;
+                a_tok[i] = p.a_rows[it.tile.row0 + r];
+            }
+        }
+    };
+    auto open_item = [&](const WorkItem &it) {
         e = it.tile.e; row0 = it.tile.row0; rows_e = it.tile.rows_e; n0 = it.tile.nt * BNO;
         b_once = __builtin_amdgcn_readfirstlane(s_tile_start[e + 1] - s_tile_start[e]) == 1;
-        s_lo = it.s_lo; S = it.s_cnt; pre = S < kStages ? S : kStages;
+        s_lo = it.s_lo; S = it.s_cnt;
         part = it.piece; split_tile = it.split_tile;
-        a_base = to_scalar((uint64_t)(uintptr_t)p.a + (uint64_t)row0 * pitch + (uint64_t)s_lo * 64);
+        pre = S < kStages ? S : kStages;
+        a_base = to_scalar((uint64_t)(uintptr_t)p.a + (GATHER ? 0 : (uint64_t)row0 * pitch) + (uint64_t)s_lo * 64);
         b_exp = to_scalar((uint64_t)(uintptr_t)p.b + (uint64_t)e * p.K * p.N * 2 +
                           (uint64_t)s_lo * (TRANS_B ? 64 : (uint64_t)kDK * p.N * 2));
 #pragma unroll
         for (int i = 0; i < CA; ++i) {
             int r = (i * NW + wave) * 16 + kc_row;
             if (r >= rows_e) r = rows_e - 1;               // clamp: loaded, never stored
-            a_off[i] = (uint32_t)r * pitch + kc_chunk * 16;
+            if constexpr (!GATHER) a_off[i] = (uint32_t)r * pitch + kc_chunk * 16;   // (GATHER: see aim_rows)
         }
         if constexpr (TRANS_B) {
 #pragma unroll
@@ -141,14 +158,23 @@ void gmm_tile256_kernel(const GmmArgs p) {
                 b_off[i] = (uint32_t)(i * 2 * NW + kn_k) * (uint32_t)p.N * 2 + (uint32_t)b_col(kn_chunk * 8) * 2;
         }
     };
+    auto open_tile = [&](long long q) {
+        const WorkItem it = locate(q);
+        fetch_rows(it);
+        open_item(it);
+    };
     // the kLoads copies of this wavefront for stage s of the item: its CA blocks of A, then its CB blocks of B
     auto issue_copies = [&](int s) {
         const uint32_t lds = smem_addr + (s % kStages) * kStage + wave * 1024;
+        // (GATHER: the compiler loses track of these wave-uniform addresses being uniform where the next item is
+        // located from inside the tile's code; to_scalar costs nothing where it has not)
+        const uint64_t a_stage = GATHER ? to_scalar(a_base + (uint64_t)s * 64) : a_base + (uint64_t)s * 64;
         static_for<0, CA>([&](auto c_tag) {
             constexpr int c = decltype(c_tag)::value;
-            copy_g2lds_16<c * kBlock>(a_off[c], a_base + (uint64_t)s * 64, lds);
+            copy_g2lds_16<c * kBlock>(a_off[c], a_stage, lds);
         });
-        const uint64_t base = b_exp + (TRANS_B ? (uint64_t)s * 64 : (uint64_t)s * kDK * p.N * 2);
+        const uint64_t b_stage = b_exp + (TRANS_B ? (uint64_t)s * 64 : (uint64_t)s * kDK * p.N * 2);
+        const uint64_t base = GATHER ? to_scalar(b_stage) : b_stage;
         if (b_once) {   // one branch per stage
             static_for<0, CB>([&](auto i_tag) {
                 constexpr int i = decltype(i_tag)::value;
@@ -159,6 +185,24 @@ void gmm_tile256_kernel(const GmmArgs p) {
                 constexpr int i = decltype(i_tag)::value;
                 copy_g2lds_16<kStageA + i * kBlock>(b_off[i], base, lds);
             });
+        }
+    };
+    // GATHER: the row numbers that fetch_rows asked for, as offsets of this lane's copies
+    uint32_t a_off_next[GATHER ? CA : 1];
+    auto aim_rows = [&]() {
+        if constexpr (GATHER) {
+#pragma unroll
+            for (int i = 0; i < CA; ++i) {
+                int tok = a_tok[i];
+                tok = tok < 0 ? 0 : (tok >= (int)p.a_src_rows ? (int)p.a_src_rows - 1 : tok);   // never outside a
+                a_off_next[i] = (uint32_t)tok * pitch + kc_chunk * 16;
+            }
+        }
+    };
+    auto take_rows = [&]() {
+        if constexpr (GATHER) {
+#pragma unroll
+            for (int i = 0; i < CA; ++i) a_off[i] = a_off_next[i];
         }
     };
     auto issue_prologue = [&]() {
@@ -211,12 +255,15 @@ void gmm_tile256_kernel(const GmmArgs p) {
     long long q = blockIdx.x;                              // the first item needs no draw (see sched_item)
     if (q < total) {
         open_tile(q);
+        aim_rows();
+        take_rows();
         issue_prologue();
     }
 
     while (q < total) {
+        WorkItem next_item{};                              // GATHER: the next item, located before this one's epilogue
         const int cur_row0 = row0, cur_rows_e = rows_e, cur_n0 = n0;
-        const int cur_part = part, cur_split_tile = split_tile;
+        const int cur_part = part, cur_split_tile = split_tile, cur_S = S;
         // 16-row fragments of this wavefront that hold at least one valid row (a short last tile skips the rest)
         int nfr = ((rows_e < kDM ? rows_e : kDM) - wm * TM + 15) / 16;
         nfr = __builtin_amdgcn_readfirstlane(nfr < 0 ? 0 : (nfr > FM ? FM : nfr));
@@ -284,6 +331,18 @@ void gmm_tile256_kernel(const GmmArgs p) {
             }
             if (kAlt && wm == 0) __syncthreads();
 
+            if constexpr (GATHER) {
+                // the next work item now, so that its row numbers travel while this tile's results are written
+                if (drawer) s_item = sched_item(draw, streams);
+                __syncthreads();
+                q = (long long)to_scalar((uint64_t)s_item);
+                if (q < total) {
+                    if (drawer) draw = sched_draw(p.sched, streams);
+                    next_item = locate(q);
+                    fetch_rows(next_item);
+                    aim_rows();
+                }
+            }
             // a piece of a split tile: its sums go to the workspace, and the piece that arrives last adds all of them up
             if (cur_part >= 0 &&
                 !meet_pieces<NW>(acc, p, plan.split, cur_split_tile, cur_part, wave, lane, kGuard ? nfr : FM))
@@ -299,7 +358,7 @@ void gmm_tile256_kernel(const GmmArgs p) {
             constexpr int RB = FNO * 32;                   // bytes per staged row
             constexpr int CPR = RB / 16;                   // lanes that write a row out
             constexpr int RPI = 64 / CPR;                  // rows per store instruction
-            char *stg = smem + (S % kStages) * kStage + wave * 4096;
+            char *stg = smem + (cur_S % kStages) * kStage + wave * 4096;
             auto swz = [](int row) { return CPR == 8 ? ((row >> 1) & 7) : ((row >> 2) & 3); };
             const int col0 = cur_n0 + (SWIGLU ? wn * (TN / 2) : wn * TN);
 #pragma unroll
@@ -337,22 +396,31 @@ void gmm_tile256_kernel(const GmmArgs p) {
         else run_tile(std::true_type{});
 
         // ---- next work item and its first copies (the stores above are older than them) ----
-        if (drawer) s_item = sched_item(draw, streams);
-        __syncthreads();   // also: the last stage has been read by everyone and the staged rows have been read back
-        q = s_item;
-        if (q < total) {
-            if (drawer) draw = sched_draw(p.sched, streams);
-            open_tile(q);
-            issue_prologue();
+        if constexpr (GATHER) {
+            __syncthreads();   // the last stage has been read by everyone and the staged rows have been read back
+            if (q < total) {
+                open_item(next_item);
+                take_rows();
+                issue_prologue();
+            }
+        } else {
+            if (drawer) s_item = sched_item(draw, streams);
+            __syncthreads();   // also: the last stage has been read by everyone and the staged rows have been read back
+            q = s_item;
+            if (q < total) {
+                if (drawer) draw = sched_draw(p.sched, streams);
+                open_tile(q);
+                issue_prologue();
+            }
         }
     }
     sched_finish(p.sched, drawer, draw, streams, total);
 }
 
-template <bool TRANS_B, bool SWIGLU>
+template <bool TRANS_B, bool SWIGLU, bool GATHER = false>
 static int launch_tile256_one(const GmmArgs &args, hipStream_t stream) {
     const size_t lds = (size_t)4 * (256 * kDK * 2 + kStageB);
-    auto kern = gmm_tile256_kernel<TRANS_B, SWIGLU>;
+    auto kern = gmm_tile256_kernel<TRANS_B, SWIGLU, GATHER>;
     static unsigned long long configured = 0;   // devices on which the kernel's LDS size has been raised
     DMOE_HIP(raise_dynamic_lds((const void *)kern, (int)lds, &configured));
     const long long grid = launch_grid(args, 256, SWIGLU, kDK, true, device_cus());

@@ -8,4 +8,7 @@ int launch_direct_bf16_256(const GmmArgs &args, bool trans_b, bool swiglu, hipSt
     return swiglu ? launch_tile256_one<false, true>(args, stream) : launch_tile256_one<false, false>(args, stream);
 }
 
+// The gate-up projection on rows fetched through args.a_rows ([K, N] weights, fused SiLU * up).
+int launch_tile256_rows(const GmmArgs &args, hipStream_t stream) { return launch_tile256_one<false, true, true>(args, stream); }
+
 }  // namespace dmoe

@@ -166,7 +166,7 @@ template <typename IdT, typename MapT, int kMode>
 __global__ __launch_bounds__(kMode == 1 ? kBlockChunks * kWave : kWave) void route_map_kernel(
     const IdT *__restrict__ ids, int64_t R, int E, int nchunks, const int *__restrict__ chunk_hist,
     const int *__restrict__ totals, int order, MapT *__restrict__ mappings, int64_t *__restrict__ batch_sizes,
-    int64_t *__restrict__ offsets) {
+    int64_t *__restrict__ offsets, int top_k, int32_t *__restrict__ row_token) {
     extern __shared__ int sm[];
     constexpr bool kSingle = kMode == 1;
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
@@ -291,6 +291,9 @@ __global__ __launch_bounds__(kMode == 1 ? kBlockChunks * kWave : kWave) void rou
             const int rank = seen + lower;
             const int pos = (order == DMOE_ORDER_REFERENCE) ? excl[id] + tot[id] - 1 - rank : excl[id] + rank;
             mappings[t] = (MapT)pos;
+            // the inverse, for a consumer that fetches the rows of a [T, d] tensor by their place in the expert-sorted
+            // order instead of having them moved there: destination row -> token
+            if (row_token != nullptr) row_token[pos] = (int32_t)((uint32_t)t / (uint32_t)top_k);
         } else if (id == -1) {
             mappings[t] = (MapT)-1;
         }
@@ -304,14 +307,14 @@ static bool one_workgroup(int64_t nchunks, int E) {
 
 template <typename IdT, typename MapT>
 static int launch_route(const void *ids, int64_t R, int E, int order, void *mappings, int64_t *batch_sizes,
-                        int64_t *offsets, void *scratch, hipStream_t stream) {
+                        int64_t *offsets, void *scratch, int top_k, int32_t *row_token, hipStream_t stream) {
     const int nchunks = (int)((R + kChunk - 1) / kChunk);
     const size_t lds = 3 * (size_t)E * sizeof(int);
     if (one_workgroup(nchunks, E)) {
         const int nw = nchunks < 1 ? 1 : nchunks;
         hipLaunchKernelGGL((route_map_kernel<IdT, MapT, 1>), dim3(1), dim3(nw * kWave), (2 + nw) * (size_t)E * sizeof(int),
                            stream, (const IdT *)ids, R, E, nw, (const int *)nullptr, (const int *)nullptr, order,
-                           (MapT *)mappings, batch_sizes, offsets);
+                           (MapT *)mappings, batch_sizes, offsets, top_k, row_token);
         DMOE_LAUNCH_CHECK("route_map_kernel");
         return DMOE_OK;
     }
@@ -328,11 +331,11 @@ static int launch_route(const void *ids, int64_t R, int E, int order, void *mapp
         DMOE_LAUNCH_CHECK("route_scan_kernel");
         hipLaunchKernelGGL((route_map_kernel<IdT, MapT, 2>), dim3(nchunks), dim3(kWave), lds, stream, (const IdT *)ids,
                            R, E, nchunks, (const int *)hist, (const int *)totals, order, (MapT *)mappings, batch_sizes,
-                           offsets);
+                           offsets, top_k, row_token);
     } else {
         hipLaunchKernelGGL((route_map_kernel<IdT, MapT, 0>), dim3(nchunks), dim3(kWave), lds, stream, (const IdT *)ids,
                            R, E, nchunks, (const int *)hist, (const int *)nullptr, order, (MapT *)mappings, batch_sizes,
-                           offsets);
+                           offsets, top_k, row_token);
     }
     DMOE_LAUNCH_CHECK("route_map_kernel");
     return DMOE_OK;
@@ -400,25 +403,43 @@ extern "C" int dmoe_route_noalloc(const void *ids, int ids_type, int64_t R, int 
     return dmoe_route(ids, ids_type, R, E, order, mappings, map_type, batch_sizes, offsets, ptr, kStaticScratchBytes, stream);
 }
 
-extern "C" int dmoe_route(const void *ids, int ids_type, int64_t R, int E, int order, void *mappings, int map_type,
-                          int64_t *batch_sizes, int64_t *offsets, void *scratch, size_t scratch_bytes,
-                          void *stream) {
+static int route_checked(const char *who, const void *ids, int ids_type, int64_t R, int E, int order, void *mappings,
+                         int map_type, int64_t *batch_sizes, int64_t *offsets, void *scratch, size_t scratch_bytes,
+                         int top_k, int32_t *row_token, void *stream) {
     size_t need = 0;
     int rc = dmoe_route_scratch_bytes(R, E, &need);
     if (rc != DMOE_OK) return rc;
     DMOE_REQUIRE(order == DMOE_ORDER_REFERENCE || order == DMOE_ORDER_STABLE, DMOE_ERR_ARG,
-                 "dmoe_route: unknown order %d", order);
-    DMOE_REQUIRE(ids_type == DMOE_I32 || ids_type == DMOE_I64, DMOE_ERR_DTYPE, "dmoe_route: ids type %d", ids_type);
-    DMOE_REQUIRE(map_type == DMOE_I32 || map_type == DMOE_I64, DMOE_ERR_DTYPE, "dmoe_route: mapping type %d",
-                 map_type);
-    DMOE_REQUIRE(R == 0 || (ids != nullptr && mappings != nullptr), DMOE_ERR_ARG, "dmoe_route: null ids/mappings");
+                 "%s: unknown order %d", who, order);
+    DMOE_REQUIRE(ids_type == DMOE_I32 || ids_type == DMOE_I64, DMOE_ERR_DTYPE, "%s: ids type %d", who, ids_type);
+    DMOE_REQUIRE(map_type == DMOE_I32 || map_type == DMOE_I64, DMOE_ERR_DTYPE, "%s: mapping type %d", who, map_type);
+    DMOE_REQUIRE(R == 0 || (ids != nullptr && mappings != nullptr), DMOE_ERR_ARG, "%s: null ids/mappings", who);
     DMOE_REQUIRE(need == 0 || (scratch != nullptr && scratch_bytes >= need), DMOE_ERR_WORKSPACE,
-                 "dmoe_route: scratch of %zu bytes needed, %zu given", need, scratch_bytes);
+                 "%s: scratch of %zu bytes needed, %zu given", who, need, scratch_bytes);
+    DMOE_REQUIRE(top_k >= 1 && R % top_k == 0, DMOE_ERR_SHAPE, "%s: R=%lld is not a multiple of top_k=%d", who, (long long)R,
+                 top_k);
     hipStream_t s = (hipStream_t)stream;
     if (ids_type == DMOE_I32) {
-        if (map_type == DMOE_I32) return launch_route<int32_t, int32_t>(ids, R, E, order, mappings, batch_sizes, offsets, scratch, s);
-        return launch_route<int32_t, int64_t>(ids, R, E, order, mappings, batch_sizes, offsets, scratch, s);
+        if (map_type == DMOE_I32)
+            return launch_route<int32_t, int32_t>(ids, R, E, order, mappings, batch_sizes, offsets, scratch, top_k, row_token, s);
+        return launch_route<int32_t, int64_t>(ids, R, E, order, mappings, batch_sizes, offsets, scratch, top_k, row_token, s);
     }
-    if (map_type == DMOE_I32) return launch_route<int64_t, int32_t>(ids, R, E, order, mappings, batch_sizes, offsets, scratch, s);
-    return launch_route<int64_t, int64_t>(ids, R, E, order, mappings, batch_sizes, offsets, scratch, s);
+    if (map_type == DMOE_I32)
+        return launch_route<int64_t, int32_t>(ids, R, E, order, mappings, batch_sizes, offsets, scratch, top_k, row_token, s);
+    return launch_route<int64_t, int64_t>(ids, R, E, order, mappings, batch_sizes, offsets, scratch, top_k, row_token, s);
+}
+
+extern "C" int dmoe_route(const void *ids, int ids_type, int64_t R, int E, int order, void *mappings, int map_type,
+                          int64_t *batch_sizes, int64_t *offsets, void *scratch, size_t scratch_bytes,
+                          void *stream) {
+    return route_checked("dmoe_route", ids, ids_type, R, E, order, mappings, map_type, batch_sizes, offsets, scratch,
+                         scratch_bytes, 1, nullptr, stream);
+}
+
+extern "C" int dmoe_route_sources(const void *ids, int ids_type, int64_t R, int E, int order, void *mappings, int map_type,
+                                  int64_t *batch_sizes, int64_t *offsets, int top_k, int32_t *row_token, void *scratch,
+                                  size_t scratch_bytes, void *stream) {
+    DMOE_REQUIRE(R == 0 || row_token != nullptr, DMOE_ERR_ARG, "dmoe_route_sources: null row_token");
+    return route_checked("dmoe_route_sources", ids, ids_type, R, E, order, mappings, map_type, batch_sizes, offsets, scratch,
+                         scratch_bytes, top_k, row_token, stream);
 }

@@ -20,16 +20,19 @@ from .ops.metadata import Metadata
 
 def expert_layer_forward(experts: torch.nn.Module, x: torch.Tensor, topk_ids: torch.Tensor,
                          topk_weights: torch.Tensor, stages: Optional[Dict[str, torch.Tensor]] = None,
-                         order: int = _lib.ORDER_REFERENCE) -> torch.Tensor:
+                         order: int = _lib.ORDER_REFERENCE, fetch_rows: Optional[bool] = None) -> torch.Tensor:
     """``x [T, d]`` bf16, ``topk_ids [T, k]`` int, ``topk_weights [T, k]`` fp32 ->
     ``[T, d]``: ``out[i] = sum_j w[i, j] * FFN_{ids[i, j]}(x[i])``.  ``stages`` (if
     given) receives the intermediate tensors of the kernels that ran; it does not change which
-    kernels run."""
+    kernels run.  ``fetch_rows``: whether the gate-up kernel fetches the tokens' rows by their
+    place in the expert-sorted order (no permute launch, no ``[R, d]`` copy of the rows; same
+    result bit for bit) instead of reading a permuted copy; ``None`` takes it where the experts
+    say it is the faster form (``MoEExperts.takes_rows``)."""
     T, k = topk_ids.shape
     num_experts = experts.num_experts
-    mappings, batch_sizes, offsets = memory.route_tokens(topk_ids, num_experts, order)
     if hasattr(experts, "forward_quantized"):
         # fp8 experts: the routed rows are quantised on their way into the expert-sorted buffer
+        mappings, batch_sizes, offsets = memory.route_tokens(topk_ids, num_experts, order)
         xq, xs = memory.permute_quantize(x, mappings)
         expert_out = experts.forward_quantized(T * k, xq, xs, batch_sizes)
         out = memory.combine_tokens(expert_out, mappings, topk_weights)
@@ -37,6 +40,17 @@ def expert_layer_forward(experts: torch.nn.Module, x: torch.Tensor, topk_ids: to
             stages.update(mappings=mappings, batch_sizes=batch_sizes, offsets=offsets, permuted_q=xq,
                           permuted_scale=xs, expert_out=expert_out)
         return out
+    if fetch_rows is None:
+        fetch_rows = hasattr(experts, "forward_rows") and x.dtype == torch.bfloat16 and experts.takes_rows(T, T * k)
+    if fetch_rows:
+        mappings, batch_sizes, offsets, row_token = memory.route_tokens_with_sources(topk_ids, num_experts, order)
+        expert_out = experts.forward_rows(x, row_token, batch_sizes)
+        out = memory.combine_tokens(expert_out, mappings, topk_weights)
+        if stages is not None:
+            stages.update(mappings=mappings, batch_sizes=batch_sizes, offsets=offsets, row_token=row_token,
+                          expert_out=expert_out)
+        return out
+    mappings, batch_sizes, offsets = memory.route_tokens(topk_ids, num_experts, order)
     permuted = memory.permute_tokens_cuda(x, mappings)
     expert_out = experts.forward(T * k, permuted, batch_sizes)
     out = memory.combine_tokens(expert_out, mappings, topk_weights)

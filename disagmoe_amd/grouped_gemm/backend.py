@@ -191,6 +191,49 @@ def gmm_swiglu(a: torch.Tensor, b: torch.Tensor, batch_sizes: torch.Tensor, tran
     return c
 
 
+def gmm_swiglu_rows(x: torch.Tensor, row_token: torch.Tensor, b: torch.Tensor, batch_sizes: torch.Tensor,
+                    c: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None,
+                    arguments_ptr: Optional[int] = None) -> torch.Tensor:
+    """:func:`gmm_swiglu` on rows fetched where they lie: row ``r`` of the product is row
+    ``row_token[r]`` of ``x [T, K]`` (``ops.memory.route_tokens_with_sources``), so the permute
+    in front of the FFN (engine.py:671-680) needs no launch.  ``b [E, K, 2I]``; returns
+    ``[R, I]``.  Runs on tiles of 256 rows whatever the batch: see :func:`takes_rows`."""
+    device = _check_operands(x, b, torch.bfloat16)
+    T, K = x.shape
+    E, Kb, N2 = b.shape
+    assert Kb == K and N2 % 2 == 0 and batch_sizes.numel() == E
+    assert row_token.dtype == torch.int32 and row_token.is_contiguous() and row_token.device == device
+    rows, inter = row_token.numel(), N2 // 2
+    if c is None:
+        c = torch.empty((rows, inter), dtype=x.dtype, device=device)
+    else:
+        assert c.is_contiguous() and c.dtype == x.dtype and c.shape[1] == inter and c.shape[0] >= rows
+    bs = _sizes_on_device(batch_sizes, device)
+    with torch.cuda.device(device):
+        _lib.call("dmoe_gmm_swiglu_rows", x.data_ptr(), row_token.data_ptr(), T, b.data_ptr(), c.data_ptr(), bs.data_ptr(),
+                  rows, E, K, inter, _lib.BF16, *_state_args(device, workspace, arguments_ptr, _stream(device)))
+    return c
+
+
+def takes_rows(T: int, rows: int, num_experts: int, K: int, inter: int) -> bool:
+    """Whether :func:`gmm_swiglu_rows` is the form to use for a gate-up projection of these
+    shapes.  It always runs the 256-row tile kernel, so it needs the library to choose that
+    kernel anyway (and the 32-bit row offsets to reach); and it has to beat the permute it
+    saves: a tile that fetches 256 scattered rows pays for them on every stage (measured on
+    MI355X: about 12 us per GB that the launch moves from the tokens to LDS, i.e. rows x K x 2
+    bytes x column tiles; 92 us on 8192 x 4096 x 14336, 19 us on 49152 x 2048 x 1408, 3 us on
+    512 x 4096 x 14336), against a permute kernel that moves (T + rows) x K x 2 bytes at about
+    5.5 TB/s behind a launch of 7 us."""
+    if K % 32 or T * K * 2 >= 1 << 32 or K * 2 * inter * 2 >= 1 << 32:
+        return False
+    if launch_plan(rows, num_experts, K, inter, swiglu=True, workspace_bytes=1 << 30)["kernel_id"] != 2:
+        return False
+    column_tiles = -(-inter // 128)
+    fetch_us = 2.0 + 12.0 * (rows * K * 2.0 * column_tiles) / 1e9
+    permute_us = 7.0 + (T + rows) * K * 2.0 / 5.5e6
+    return fetch_us < permute_us
+
+
 def get_arguments(num_experts: int, device: torch.device) -> Tuple[int, int]:
     """``(workspace_size, arguments_ptr)`` as in experts.py:69-72 and
     tests/ops/test_gemm.py:24.  ``arguments_ptr`` is the address of a zeroed state

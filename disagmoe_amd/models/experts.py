@@ -109,6 +109,19 @@ class MoEExperts(_GemmState, torch.nn.Module):
         h = gg.gmm_swiglu(hiddens, self.w13_weight, batch_sizes, **ws)
         return gg.gmm(h, self.w2_weight, batch_sizes, **ws)
 
+    def forward_rows(self, x: torch.Tensor, row_token: torch.Tensor, batch_sizes: torch.Tensor) -> torch.Tensor:
+        """:meth:`forward` on rows that are fetched where they lie: ``x [T, d]`` in token order
+        and ``row_token [R]`` (``ops.memory.route_tokens_with_sources``) instead of the
+        expert-sorted copy ``hiddens [R, d]``: the gate-up kernel reads row ``row_token[r]`` of
+        ``x``, and the permute in front of the FFN (engine.py:671-680) is never launched."""
+        ws = self._gemm_state()
+        h = gg.gmm_swiglu_rows(x, row_token, self.w13_weight, batch_sizes, **ws)
+        return gg.gmm(h, self.w2_weight, batch_sizes, **ws)
+
+    def takes_rows(self, T: int, rows: int) -> bool:
+        """Whether :meth:`forward_rows` is the faster form for a batch of these sizes."""
+        return gg.takes_rows(T, rows, self.num_experts, self.hidden_size, self.intermediate_size)
+
     def forward_unfused(self, bs: int, hiddens: torch.Tensor, batch_sizes: torch.Tensor) -> torch.Tensor:
         """The reference's own schedule, statement by statement (experts.py:92-94):
         the gate-up result, SiLU and the product are each rounded to bf16."""

@@ -75,6 +75,32 @@ def route_tokens(exp_ids: torch.Tensor, num_experts: int, order: int = _lib.ORDE
     return mappings, batch_sizes, offsets
 
 
+def route_tokens_with_sources(topk_ids: torch.Tensor, num_experts: int, order: int = _lib.ORDER_REFERENCE,
+                              map_dtype: torch.dtype = torch.int64):
+    """:func:`route_tokens` of ``topk_ids [T, k]`` that also returns ``row_token [R]`` int32, the token
+    whose row stands at each place of the expert-sorted order (``row_token[mappings[i*k + j]] = i``):
+    what ``grouped_gemm.backend.gmm_swiglu_rows`` fetches its rows by."""
+    device = _device_of(topk_ids)
+    assert topk_ids.dim() == 2
+    k = topk_ids.shape[1]
+    ids = topk_ids.to(device).contiguous().view(-1)
+    if ids.dtype not in _INT_TYPES:
+        raise TypeError(f"expert ids must be int32 or int64, got {ids.dtype}")
+    R = ids.numel()
+    with torch.cuda.device(device):
+        need = _lib.c_size_t(0)
+        _lib.call("dmoe_route_scratch_bytes", R, num_experts, _lib.ctypes.byref(need))
+        mappings = torch.empty(R, dtype=map_dtype, device=device)
+        batch_sizes = torch.empty(num_experts, dtype=torch.int64, device=device)
+        offsets = torch.empty(num_experts + 1, dtype=torch.int64, device=device)
+        row_token = torch.empty(R, dtype=torch.int32, device=device)
+        scratch = torch.empty(max(need.value, 1), dtype=torch.uint8, device=device)
+        _lib.call("dmoe_route_sources", ids.data_ptr(), _INT_TYPES[ids.dtype], R, num_experts, order, mappings.data_ptr(),
+                  _INT_TYPES[map_dtype], batch_sizes.data_ptr(), offsets.data_ptr(), k, row_token.data_ptr(),
+                  scratch.data_ptr(), scratch.numel(), _stream(device))
+    return mappings, batch_sizes, offsets, row_token
+
+
 def get_mappings_from_exp_ids(exp_ids: Union[torch.Tensor, List[int]], num_experts: int) -> Tuple[List[int], List[int]]:
     """Reference signature and return types (memory.py:34-54): Python lists
     ``(mappings, exp_cnt)``.  Ids that live on the host (a list, as the reference's

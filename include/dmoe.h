@@ -78,6 +78,15 @@ int dmoe_route(const void *ids, int ids_type, int64_t R, int E, int order,
                void *mappings, int map_type, int64_t *batch_sizes, int64_t *offsets,
                void *scratch, size_t scratch_bytes, void *stream);
 
+/* dmoe_route that also writes the inverse of the mapping in tokens: row_token[mappings[t]] = t / top_k, int32 [R]
+ * (ids with an expert outside [0, E) leave no entry).  For dmoe_gmm_swiglu_rows, which fetches the rows of the
+ * [T, d] activations by their place in the expert-sorted order, so that the duplicating permute of
+ * disagmoe/frontend/engine.py:671-680 (permute_tokens_cuda before the FFN) needs no launch of its own.
+ * R % top_k == 0. */
+int dmoe_route_sources(const void *ids, int ids_type, int64_t R, int E, int order,
+                       void *mappings, int map_type, int64_t *batch_sizes, int64_t *offsets,
+                       int top_k, int32_t *row_token, void *scratch, size_t scratch_bytes, void *stream);
+
 /* dmoe_route for callers that cannot allocate device memory (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in
  * the reference.  Same arguments and results as dmoe_route without the scratch
@@ -248,6 +257,16 @@ int dmoe_gmm(const void *a, const void *b, void *c, const int64_t *batch_sizes,
 int dmoe_gmm_swiglu(const void *a, const void *b, void *h, const int64_t *batch_sizes,
                     int64_t rows, int E, int64_t K, int64_t I, int trans_b, int dtype,
                     void *state, void *workspace, size_t workspace_bytes, void *stream);
+
+/* dmoe_gmm_swiglu on rows that are fetched where they lie: row r of the product is row row_token[r] of x [T, K]
+ * (dmoe_route_sources writes row_token).  The duplicating permute in front of the FFN
+ * (disagmoe/frontend/engine.py:671-680, csrc/cuda_ops/permute.cu:86-112) and the gather of
+ * TensorBatch::merge (csrc/include/datatypes.hpp:508-549) then need no launch and no copy of the rows.
+ * Weights [E, K, 2I]; K % 32 == 0; T * K * 2 and K * 2I * 2 below 4 GiB.  Always runs on tiles of 256 rows:
+ * for problems whose rows do not fill such tiles, dmoe_permute + dmoe_gmm_swiglu is the faster pair. */
+int dmoe_gmm_swiglu_rows(const void *x, const int32_t *row_token, int64_t T, const void *b, void *h,
+                         const int64_t *batch_sizes, int64_t rows, int E, int64_t K, int64_t I, int dtype,
+                         void *state, void *workspace, size_t workspace_bytes, void *stream);
 
 /* ---- fp8 (e4m3) path: no counterpart in the reference ---------------------
  * Per-row quantisation: q[r, :] = fp8(x[r, :] / s[r]), s[r] = absmax(x[r, :]) / 448

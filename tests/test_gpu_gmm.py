@@ -319,6 +319,40 @@ def test_cut_launches_alternating_operands_on_one_state(variant, swiglu):
     gg.set_tile_variant(0)
 
 
+@pytest.mark.parametrize("T,k,E,K,I", [(300, 2, 8, 256, 384), (1000, 1, 3, 1024, 128), (512, 6, 64, 512, 256),
+                                        (64, 2, 8, 8192, 256), (2048, 2, 4, 96, 136)])
+def test_gmm_swiglu_rows_equals_permute_then_gmm(T, k, E, K, I):
+    # The gate-up projection that fetches the tokens' rows by their place in the expert-sorted order against the pair
+    # it replaces (permute, then the same kernel on the copy): the same bits, and the oracle's values.  Experts without
+    # rows, experts of a few rows, a long K whose tiles are cut in pieces (one state block and workspace for both).
+    from disagmoe_amd.ops import memory
+    announce(test="gmm_swiglu_rows", T=T, k=k, E=E, K=K, I=I)
+    g = torch.Generator().manual_seed(T + K)
+    x = torch.randn(T, K, generator=g).to(torch.bfloat16)
+    w13 = (torch.randn(E, K, 2 * I, generator=g) * 0.05).to(torch.bfloat16)
+    ids = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(torch.int32)
+    if E > 2:
+        ids[ids == 1] = 2 if k == 1 else ids[ids == 1]                # (top-1: an expert without rows)
+    m, bs, off, row_token = memory.route_tokens_with_sources(ids.to(dev()), E)
+    assert torch.equal(row_token.cpu().long(), torch.argsort(m.cpu()) // k)
+    m0, bs0, off0 = memory.route_tokens(ids.to(dev()), E)
+    assert torch.equal(m, m0) and torch.equal(bs, bs0) and torch.equal(off, off0)
+    xp = memory.permute_tokens_cuda(x.to(dev()), m)
+    size, ptr = gg.get_arguments(E, dev())
+    workspace = torch.empty([size], dtype=torch.uint8, device=dev())
+    gg.set_tile_variant(7)                                            # the kernel that the row-fetching form runs on
+    want = gg.gmm_swiglu(xp, w13.to(dev()), bs, workspace=workspace, arguments_ptr=ptr)
+    gg.set_tile_variant(0)
+    got = gg.gmm_swiglu_rows(x.to(dev()), row_token, w13.to(dev()), bs, workspace=workspace, arguments_ptr=ptr)
+    again = gg.gmm_swiglu_rows(x.to(dev()), row_token, w13.to(dev()), bs, workspace=workspace, arguments_ptr=ptr)
+    torch.cuda.synchronize()
+    assert torch.equal(got, want) and torch.equal(again, want)
+    u = ffn.gmm(xp.cpu(), w13, bs.cpu(), out_dtype=torch.float32)
+    ref = (torch.nn.functional.silu(u[:, :I]) * u[:, I:]).to(torch.bfloat16)
+    assert max_rel_err(got, ref) <= TOL_BF16
+    assert int(gg._STATE_BLOCKS[ptr].count_nonzero()) == 0
+
+
 def test_gmm_launches_on_two_streams_keep_their_own_state():
     # a recorded graph of a layer (its own state block and workspace) is replayed on one stream while 80 eager launches
     # with the module-wide pair of another stream run beside it; both give the bits of their serial runs

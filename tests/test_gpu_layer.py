@@ -40,7 +40,12 @@ def test_c1_full_layer_against_oracle():
     w13, w2 = workloads.make_weights(w, "cpu")
     layer = _layer_from(w13.to(dev()), w2.to(dev()))
     stages = {}
-    out = expert_layer_forward(layer, x.to(dev()), ids.to(dev()), gates.to(dev()), stages=stages)
+    out = expert_layer_forward(layer, x.to(dev()), ids.to(dev()), gates.to(dev()), stages=stages, fetch_rows=False)
+    # the form without a permute launch (the gate-up kernel fetches the tokens' rows itself): the same bits
+    st2 = {}
+    out2 = expert_layer_forward(layer, x.to(dev()), ids.to(dev()), gates.to(dev()), stages=st2, fetch_rows=True)
+    assert torch.equal(out2, out) and torch.equal(st2["expert_out"], stages["expert_out"])
+    assert torch.equal(st2["row_token"].cpu().long(), torch.argsort(stages["mappings"].cpu()) // w.k)
     m_ref, cnt = routing.get_mappings_from_exp_ids(ids, w.E)
     assert stages["mappings"].cpu().tolist() == m_ref and stages["batch_sizes"].cpu().tolist() == cnt
     from oracle import rows
@@ -63,7 +68,10 @@ def test_full_size_layer(name, rows_per_expert):
     w13, w2 = workloads.make_weights(w, dev())
     layer = _layer_from(w13, w2)
     stages = {}
-    out = expert_layer_forward(layer, x, ids.to(dev()), gates.to(dev()), stages=stages)
+    out = expert_layer_forward(layer, x, ids.to(dev()), gates.to(dev()), stages=stages, fetch_rows=False)
+    # the default form for these sizes, which may leave the permute to the gate-up kernel: the same bits
+    assert torch.equal(expert_layer_forward(layer, x, ids.to(dev()), gates.to(dev())), out)
+    assert torch.equal(expert_layer_forward(layer, x, ids.to(dev()), gates.to(dev()), fetch_rows=True), out)
     torch.cuda.synchronize()
     m_ref, cnt = routing.get_mappings_from_exp_ids(ids, w.E)
     assert stages["mappings"].cpu().tolist() == m_ref and stages["batch_sizes"].cpu().tolist() == cnt

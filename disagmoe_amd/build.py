@@ -14,7 +14,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_PATH = os.path.join(HERE, "libdmoe_hip.so")
-SOURCES = ["gmm_wave128.hip", "gmm_tile256.hip", "gmm_tile256_fp8.hip", "gmm_direct_bf16.hip", "gmm_direct_bf16_small.hip", "gmm_direct_fp8.hip", "gmm.hip", "route.hip", "topk.hip", "rows.hip",
+SOURCES = ["gmm_wave128_fp8.hip", "gmm_wave128.hip", "gmm_tile256.hip", "gmm_tile256_fp8.hip", "gmm_direct_bf16.hip", "gmm_direct_bf16_small.hip", "gmm_direct_fp8.hip", "gmm.hip", "route.hip", "topk.hip", "rows.hip",
            "meta.hip"]
 ARCH = "gfx950"
 

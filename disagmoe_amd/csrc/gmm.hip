@@ -515,6 +515,8 @@ static GmmLaunch choose_launch(const GmmArgs &args, bool trans_b, bool swiglu, b
             L.kernel = kKernelWave128; L.waves = 4;
         } else if (tile_rows == 256 && !fp8) {
             L.kernel = kKernelTile256; L.waves = 8;
+        } else if (tile_rows == 256 && args.K % 128 == 0 && g_variant == 8) {
+            L.kernel = kKernelWave128Fp8; L.waves = 4;
         } else if (tile_rows == 256 && args.K % 128 == 0) {
             L.kernel = kKernelTile256Fp8; L.waves = 8;   // whole k-steps of 128: the tile that copies whole 128-byte lines
         } else {
@@ -539,6 +541,7 @@ static int launch_by_rows(const GmmArgs &args, hipStream_t stream) {
         return launch_one<256, 256, 2, 4, TRANS_B, SWIGLU, FP8>(args, stream);
     }
     if (L.kernel == kKernelWave128) return launch_wave128(args, SWIGLU, stream);
+    if (L.kernel == kKernelWave128Fp8) return launch_wave128_fp8(args, SWIGLU, stream);
     if constexpr (FP8) return launch_direct_fp8(args, L.tile_rows, SWIGLU, stream);
     else return launch_direct_bf16(args, L.tile_rows, TRANS_B, SWIGLU, stream);
 }

@@ -322,7 +322,7 @@ __device__ __forceinline__ bool meet_pieces(AccT (&acc)[FM][FN], const GmmArgs &
 }
 
 // ---- the launch a problem gets (host) -------------------------------------------------------------------
-enum GmmKernelId { kKernelStaged = 0, kKernelDirect = 1, kKernelTile256 = 2, kKernelTile256Fp8 = 3, kKernelWave128 = 4 };
+enum GmmKernelId { kKernelStaged = 0, kKernelDirect = 1, kKernelTile256 = 2, kKernelTile256Fp8 = 3, kKernelWave128 = 4, kKernelWave128Fp8 = 5 };
 struct GmmLaunch {
     int kernel;        // GmmKernelId
     int tile_rows;     // rows of a tile (64, 128, 256); a tile has 256 columns of b
@@ -350,6 +350,7 @@ int launch_direct_bf16(const GmmArgs &args, int tile_rows, bool trans_b, bool sw
 int launch_direct_fp8(const GmmArgs &args, int tile_rows, bool swiglu, hipStream_t stream);
 int launch_tile256_fp8(const GmmArgs &args, bool swiglu, hipStream_t stream);
 int launch_wave128(const GmmArgs &args, bool swiglu, hipStream_t stream);
+int launch_wave128_fp8(const GmmArgs &args, bool swiglu, hipStream_t stream);
 int launch_tile256_rows(const GmmArgs &args, hipStream_t stream);
 
 }  // namespace dmoe

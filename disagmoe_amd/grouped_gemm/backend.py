@@ -106,7 +106,7 @@ def release_arguments(arguments_ptr: int) -> None:
 
 
 KERNEL_NAMES = {0: "dmoe::gmm_kernel", 1: "dmoe::gmm_direct_kernel", 2: "dmoe::gmm_tile256_kernel",
-                3: "dmoe::gmm_tile256_fp8_kernel", 4: "dmoe::gmm_wave128_kernel"}
+                3: "dmoe::gmm_tile256_fp8_kernel", 4: "dmoe::gmm_wave128_kernel", 5: "dmoe::gmm_wave128_fp8_kernel"}
 
 
 def launch_plan(rows: int, num_experts: int, K: int, N: int, swiglu: bool = False, fp8: bool = False,

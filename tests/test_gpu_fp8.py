@@ -51,7 +51,7 @@ def test_quantize_weight_matches_oracle():
     assert torch.equal(s.cpu(), s_ref) and torch.equal(q.cpu().view(torch.uint8), q_ref.view(torch.uint8))
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, 8])
 @pytest.mark.parametrize("E,R,K,N", [(1, 200, 256, 256), (4, 1000, 512, 520), (8, 700, 144, 264), (3, 1300, 320, 384)])
 def test_gmm_fp8(variant, E, R, K, N):
     announce(test="gmm_fp8", variant=variant, E=E, R=R, K=K, N=N)
@@ -78,7 +78,7 @@ def test_gmm_fp8(variant, E, R, K, N):
         gg.set_tile_variant(0)
 
 
-@pytest.mark.parametrize("variant,R", [(0, 600), (5, 600), (6, 600), (7, 600), (0, 1900)])
+@pytest.mark.parametrize("variant,R", [(0, 600), (5, 600), (6, 600), (7, 600), (8, 600), (0, 1900)])
 def test_fp8_experts_forward(variant, R):
     # variants 5, 6, 7: the 64-, 128- and 256-row tiles of the default kernels; 1900 rows pick the 256-row tile by themselves
     announce(test="fp8_experts_forward", variant=variant, R=R)
@@ -185,6 +185,7 @@ def test_gmm_fp8_few_stages(variant, K):
         gg.set_tile_variant(0)
 
 
+@pytest.mark.parametrize("variant", [7, 8])
 @pytest.mark.parametrize("swiglu", [False, True])
 @pytest.mark.parametrize("K,N,sizes", [
     (128, 256, [256, 0, 1, 255, 257]),                 # one k-step; full, empty, 1-row, 255-row tiles and a 1-row last tile
@@ -194,10 +195,12 @@ def test_gmm_fp8_few_stages(variant, K):
     (3200, 512, [500, 0, 290]),                        # fewer tiles than compute units
     (8320, 512, [500, 0, 290]),                        # ... and a long K: cut along K in uneven pieces (65 k-steps)
 ])
-def test_gmm_fp8_tile_of_whole_lines(K, N, sizes, swiglu):
-    """The 256-row fp8 tile whose copies fetch whole 128-byte lines (K % 128 == 0; variant 7 picks 256-row tiles)."""
-    announce(test="gmm_fp8_tile_of_whole_lines", K=K, N=N, sizes=sizes, swiglu=swiglu)
-    gg.set_tile_variant(7)
+def test_gmm_fp8_tile_of_whole_lines(K, N, sizes, swiglu, variant):
+    """The 256-row fp8 tiles that move whole 128-byte lines (K % 128 == 0): variant 7 picks the one on 8 wavefronts with
+    copies straight into LDS, variant 8 the one on 4 wavefronts of 128 x 128 with operands staged through registers.
+    Both add up the same k-steps in the same order with the same instruction: their results are equal bit for bit."""
+    announce(test="gmm_fp8_tile_of_whole_lines", K=K, N=N, sizes=sizes, swiglu=swiglu, variant=variant)
+    gg.set_tile_variant(variant)
     try:
         E, R = len(sizes), sum(sizes)
         n_w = 2 * N if swiglu else N
@@ -217,6 +220,10 @@ def test_gmm_fp8_tile_of_whole_lines(K, N, sizes, swiglu):
         assert max_rel_err(out, exact) <= 1e-2, max_rel_err(out, exact)
         again = run(aq.to(dev()), a_s.to(dev()), wq.to(dev()), w_s.to(dev()), bs)
         assert torch.equal(out, again)                 # pieces are summed in a fixed order
+        if variant == 8:
+            gg.set_tile_variant(7)
+            other = run(aq.to(dev()), a_s.to(dev()), wq.to(dev()), w_s.to(dev()), bs)
+            assert torch.equal(out, other)
     finally:
         gg.set_tile_variant(0)
 
@@ -237,13 +244,14 @@ def _fp8_case(K, N, sizes, swiglu, seed):
     return (aq.to(dev()), a_s.to(dev()), wq.to(dev()), w_s.to(dev()), bs.to(dev())), exact
 
 
+@pytest.mark.parametrize("variant", [7, 8])
 @pytest.mark.parametrize("swiglu", [False, True])
-def test_fp8_cut_launches_alternating_operands_on_one_state(swiglu):
-    """Two different problems A, B, A, B, ... through launches of the 256-row fp8 tile that cut their tiles along K, on
+def test_fp8_cut_launches_alternating_operands_on_one_state(swiglu, variant):
+    """Two different problems A, B, A, B, ... through launches of the 256-row fp8 tiles that cut their tiles along K, on
     one state block and one workspace: what a launch leaves there (or a stale copy of it in a cache) belongs to other
     operands than the next launch's.  Every result against the oracle and against the uncut launch."""
-    announce(test="fp8_split_alternating", swiglu=swiglu)
-    gg.set_tile_variant(7)
+    announce(test="fp8_split_alternating", swiglu=swiglu, variant=variant)
+    gg.set_tile_variant(variant)
     try:
         K, N = 8192, 512
         cases = [_fp8_case(K, N, [500, 0, 290], swiglu, 21), _fp8_case(K, N, [260, 300, 200], swiglu, 22)]
@@ -252,7 +260,7 @@ def test_fp8_cut_launches_alternating_operands_on_one_state(swiglu):
         workspace = torch.empty([size], dtype=torch.uint8, device=dev())
         for ops, _ in cases:
             plan = gg.launch_plan(int(ops[4].sum()), 3, K, N, swiglu=swiglu, fp8=True, workspace_bytes=size, batch_sizes=ops[4].cpu())
-            assert plan["kernel_id"] == 3 and plan["pieces_per_cut_tile"] > 1, plan
+            assert plan["kernel_id"] == (3 if variant == 7 else 5) and plan["pieces_per_cut_tile"] > 1, plan
         uncut = [run(*ops, arguments_ptr=ptr) for ops, _ in cases]
         outs = [run(*cases[rep % 2][0], workspace=workspace, arguments_ptr=ptr) for rep in range(6)]
         torch.cuda.synchronize()

@@ -153,6 +153,20 @@ void gmm_tile256_fp8_kernel(const GmmArgs p) {
         issue_prologue();
     }
 
+    // Ticks of the 100 MHz clock that a k-step of this workgroup's full tiles takes (0: none finished yet).  A tile with
+    // fewer than 256 rows skips the MFMAs of its empty row fragments; left to itself it walks K faster than the tiles
+    // beside it that share its weight tile, ends early, and from then on its workgroup draws every tile ahead of its
+    // neighbours: the compute units of an XCD fall out of step for the rest of the launch and what they share in
+    // principle no longer meets in the 4 MB of their L2 (measured on 8 experts of 4031 .. 4143 rows, K = 6144: tiles
+    // start within 2 us of each other inside an XCD until the first short tiles, 26 us apart behind them and 113 us at
+    // the end; the launch fetches 6 times its operands).  So a short tile holds the pace of a full one: the first
+    // wavefront waits at the end of every k-step until a full tile would be there (the others wait at the barrier; a
+    // wait on a clock, so it always ends).  With that the tiles of an XCD start within 4.4 us of each other to the end
+    // of the launch and it fetches 10.0 GB instead of 17.9 GB at the same speed (2736 - 2777 against 2749 - 2774
+    // TFLOP/s in alternating runs).  Only in the fused launch: the plain product of the same rows (K = 16384, N = 6144)
+    // fetches 5.7 GB instead of 7.9 GB that way but runs 1.5 % slower, the idle time of its short tiles being worth
+    // more than the traffic.
+    long long full_step_ticks = 0;
     while (q < total) {
         const int cur_row0 = row0, cur_rows_e = rows_e, cur_n0 = n0, cur_e = e;
         const int cur_part = part, cur_split_tile = split_tile;
@@ -170,6 +184,9 @@ void gmm_tile256_fp8_kernel(const GmmArgs p) {
             // the early group of k-step 0 has landed (its late group and k-step 1 may be in flight)
             if (T > 1) DMOE_WAIT_VMCNT(kLate + kEarly + kLate); else DMOE_WAIT_VMCNT(kLate);
             __syncthreads();
+            const bool short_tile = cur_rows_e < kDM;
+            const bool pace = SWIGLU && short_tile && full_step_ticks > 0 && wave == 0;
+            const long long t_begin = (long long)wall_clock64();
             // Phases of k-step t, for the early half of the wavefronts (the late half one phase later): memory a (the B
             // fragments, row fragments 0 - 3), matrix a, memory b (row fragments 4 - 7), matrix b.  What memory a reads is
             // free once the late half has left its memory a, so memory b of k-step t issues the early group of k-step
@@ -216,6 +233,10 @@ void gmm_tile256_fp8_kernel(const GmmArgs p) {
                     if (h == 0) landed_late(t);
                     else if (next) landed_early(t);
                 }
+                if (h == 1 && pace) {
+                    const long long due = t_begin + (long long)(t + 1) * full_step_ticks;
+                    while ((long long)wall_clock64() < due) __builtin_amdgcn_s_sleep(2);
+                }
                 __builtin_amdgcn_sched_barrier(0);
                 __syncthreads();
                 __builtin_amdgcn_sched_barrier(0);
@@ -226,6 +247,7 @@ void gmm_tile256_fp8_kernel(const GmmArgs p) {
                 half_step(t, std::integral_constant<int, 1>{}, t + 1 < T);
             }
             if (wm == 0) __syncthreads();
+            if (!short_tile && wave == 0) full_step_ticks = ((long long)wall_clock64() - t_begin) / T;
 
             // a piece of a split tile: its sums go to the workspace, and the piece that arrives last adds all of them up
             if (cur_part >= 0 &&

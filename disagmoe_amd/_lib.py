@@ -44,25 +44,25 @@ SIGNATURES = {
     "dmoe_combine": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int64, c_int, c_int64, c_int, c_int,
                              c_void_p]),
     "dmoe_gmm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int64, c_int64, c_int, c_int,
-                         c_void_p, c_void_p, c_size_t, c_void_p]),
+                         c_void_p, c_void_p, c_size_t, c_void_p, c_void_p]),
     "dmoe_gmm_swiglu": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int64, c_int64, c_int,
-                                c_int, c_void_p, c_void_p, c_size_t, c_void_p]),
+                                c_int, c_void_p, c_void_p, c_size_t, c_void_p, c_void_p]),
     "dmoe_gmm_swiglu_rows": (c_int, [c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int64,
-                                     c_int64, c_int, c_void_p, c_void_p, c_size_t, c_void_p]),
+                                     c_int64, c_int, c_void_p, c_void_p, c_size_t, c_void_p, c_void_p]),
     "dmoe_gmm_workspace_bytes": (c_int, [c_int, POINTER(c_size_t)]),
     "dmoe_quant_rows": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int, c_void_p]),
     "dmoe_permute_quant": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int,
                                    c_void_p]),
     "dmoe_gmm_fp8": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int64,
-                             c_int64, c_void_p, c_void_p, c_size_t, c_void_p]),
+                             c_int64, c_void_p, c_void_p, c_size_t, c_void_p, c_void_p]),
     "dmoe_gmm_fp8_swiglu": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int,
-                                    c_int64, c_int64, c_void_p, c_void_p, c_size_t, c_void_p]),
+                                    c_int64, c_int64, c_void_p, c_void_p, c_size_t, c_void_p, c_void_p]),
 }
 
 #: exported for the library's own tests and benchmarks, not declared in include/dmoe.h (csrc/tuning.h)
 TEST_HOOKS = {
     "dmoe_gmm_tune": (c_int, [c_int]),
-    "dmoe_gmm_plan": (c_int, [c_void_p, c_int64, c_int, c_int64, c_int64, c_int, c_int, c_int, c_size_t, c_void_p]),
+    "dmoe_gmm_plan": (c_int, [c_void_p, c_int, c_int64, c_int, c_int64, c_int64, c_int, c_int, c_int, c_size_t, c_void_p]),
 }
 GMM_STATE_BYTES = 33024
 

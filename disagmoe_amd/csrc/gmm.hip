@@ -406,6 +406,14 @@ static int launch_one(const GmmArgs &args, hipStream_t stream) {
 }
 
 static int g_variant = 0;  // tuning hook, see dmoe_gmm_tune
+thread_local const int64_t *t_host_sizes = nullptr;
+namespace {
+// the host copy of the sizes for the length of one call
+struct HostSizes {
+    explicit HostSizes(const int64_t *p) { t_host_sizes = p; }
+    ~HostSizes() { t_host_sizes = nullptr; }
+};
+}  // namespace
 
 // ---- where a launch keeps its counters ----------------------------------------------------------------
 // With a state block of the caller: there, the split tiles' arrival counters behind them, and the partial sums in
@@ -489,9 +497,19 @@ static GmmLaunch choose_launch(const GmmArgs &args, bool trans_b, bool swiglu, b
         // small batch on few experts: 176 half-filled tall tiles instead of 264: 12 % off that launch).  Else the rows
         // per expert on average decide, and a size that would leave more than half of the CUs without a tile is halved
         // (small problems: latency counts).
-        const long long avg = args.rows / (args.E > 0 ? args.E : 1);
+        // With the sizes on the host the tiles of every height are counted, and the rows per expert are those of the
+        // experts that have any (a skewed decode batch: a few experts hold most of the rows); without, estimated.
+        long long busy = args.E > 0 ? args.E : 1;
+        if (t_host_sizes != nullptr) {
+            busy = 0;
+            for (int e = 0; e < args.E; ++e) busy += t_host_sizes[e] > 0;
+            if (busy < 1) busy = 1;
+        }
+        const long long avg = args.rows / busy;
         const long long n_tiles = ((swiglu ? args.N / 2 : args.N) + (swiglu ? 127 : 255)) / (swiglu ? 128 : 256);
-        const long long est256 = (args.rows / 256 + (args.E + 1) / 2) * n_tiles, est128 = (args.rows / 128 + (args.E + 1) / 2) * n_tiles;
+        const bool exact = t_host_sizes != nullptr;
+        const long long est256 = (exact ? m_tiles_of(args, 256) : args.rows / 256 + (args.E + 1) / 2) * n_tiles;
+        const long long est128 = (exact ? m_tiles_of(args, 128) : args.rows / 128 + (args.E + 1) / 2) * n_tiles;
         // fp8: the 256-row tile copies whole 128-byte lines (gmm_tile256_fp8.h) and streams weights a third faster than
         // the smaller tiles, which copy half lines (decode-sized batch, K 4096, N 28672: 4.1 against 3.2 TB/s); it is
         // taken wherever its tiles fill half of the CUs (a quarter, where the launch may cut its tiles along a long K
@@ -501,7 +519,8 @@ static GmmLaunch choose_launch(const GmmArgs &args, bool trans_b, bool swiglu, b
         int tile_rows = 256;
         if (!tall) {
             tile_rows = avg <= 64 ? 64 : (avg <= 160 ? 128 : 256);
-            while (tile_rows > 64 && (args.rows / tile_rows + (args.E + 1) / 2) * n_tiles * 2 < cus) tile_rows /= 2;
+            while (tile_rows > 64 && (exact ? m_tiles_of(args, tile_rows) : args.rows / tile_rows + (args.E + 1) / 2) * n_tiles * 2 < cus)
+                tile_rows /= 2;
         }
         if (g_variant >= 5) tile_rows = g_variant == 5 ? 64 : (g_variant == 6 ? 128 : 256);   // test hook: fixed tile rows (7, 8: 256)
         L.tile_rows = tile_rows;
@@ -578,8 +597,10 @@ extern "C" int dmoe_gmm_tune(int variant) {
 // What a launch with these shapes would run (see tuning.h).  out: [0] kernel (GmmKernelId), [1] tile rows, [2] wavefronts
 // per workgroup, [3] workgroups, [4] k per stage unit; and, when the sizes are given (host memory), what the kernel
 // derives from them on the device: [5] tiles, [6] tiles cut along K, [7] pieces per cut tile, [8] work items; -1 without.
-extern "C" int dmoe_gmm_plan(const int64_t *host_batch_sizes, int64_t rows, int E, int64_t K, int64_t N, int trans_b,
-                             int swiglu, int dtype, size_t workspace_bytes, int64_t *out) {
+// `launch_has_sizes`: the launch in question is given the host sizes too (host_batch_sizes of dmoe_gmm*), so its tile
+// height and grid are decided from them; otherwise the sizes only serve the counts [5] .. [8].
+extern "C" int dmoe_gmm_plan(const int64_t *host_batch_sizes, int launch_has_sizes, int64_t rows, int E, int64_t K, int64_t N,
+                             int trans_b, int swiglu, int dtype, size_t workspace_bytes, int64_t *out) {
     DMOE_REQUIRE(out != nullptr, DMOE_ERR_ARG, "dmoe_gmm_plan: null output");
     DMOE_REQUIRE(dtype == DMOE_BF16 || dtype == DMOE_FP8_E4M3, DMOE_ERR_DTYPE, "dmoe_gmm_plan: dtype %d", dtype);
     const bool fp8 = dtype == DMOE_FP8_E4M3;
@@ -589,6 +610,7 @@ extern "C" int dmoe_gmm_plan(const int64_t *host_batch_sizes, int64_t rows, int 
     GmmArgs args{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, rows, E, (int)K, (int)n_cols, (int)N};
     args.arrive = workspace_bytes > 0 ? (unsigned int *)out : nullptr;   // only tested against nullptr
     args.partial_bytes = (long long)workspace_bytes;
+    const HostSizes known(launch_has_sizes ? host_batch_sizes : nullptr);
     const GmmLaunch L = choose_launch(args, trans_b != 0 || fp8, swiglu != 0, fp8);
     out[0] = L.kernel; out[1] = L.tile_rows; out[2] = L.waves; out[3] = L.grid; out[4] = L.stage_k;
     out[5] = out[6] = out[7] = out[8] = -1;
@@ -626,7 +648,8 @@ extern "C" int dmoe_gmm_workspace_bytes(int E, size_t *bytes) {
 
 extern "C" int dmoe_gmm(const void *a, const void *b, void *c, const int64_t *batch_sizes, int64_t rows, int E,
                         int64_t K, int64_t N, int trans_b, int dtype, void *state, void *workspace,
-                        size_t workspace_bytes, void *stream) {
+                        size_t workspace_bytes, const int64_t *host_batch_sizes, void *stream) {
+    const HostSizes known(host_batch_sizes);
     DMOE_REQUIRE(dtype == DMOE_BF16, DMOE_ERR_DTYPE, "dmoe_gmm: dtype %d (bf16 only)", dtype);
     int rc = check_gmm("dmoe_gmm", a, b, c, batch_sizes, rows, E, K, N, 8);
     if (rc != DMOE_OK) return rc;
@@ -640,7 +663,8 @@ extern "C" int dmoe_gmm(const void *a, const void *b, void *c, const int64_t *ba
 
 extern "C" int dmoe_gmm_swiglu(const void *a, const void *b, void *h, const int64_t *batch_sizes, int64_t rows, int E,
                                int64_t K, int64_t I, int trans_b, int dtype, void *state, void *workspace,
-                               size_t workspace_bytes, void *stream) {
+                               size_t workspace_bytes, const int64_t *host_batch_sizes, void *stream) {
+    const HostSizes known(host_batch_sizes);
     DMOE_REQUIRE(dtype == DMOE_BF16, DMOE_ERR_DTYPE, "dmoe_gmm_swiglu: dtype %d (bf16 only)", dtype);
     int rc = check_gmm("dmoe_gmm_swiglu", a, b, h, batch_sizes, rows, E, K, I, 8);
     if (rc != DMOE_OK) return rc;
@@ -654,7 +678,9 @@ extern "C" int dmoe_gmm_swiglu(const void *a, const void *b, void *h, const int6
 
 extern "C" int dmoe_gmm_swiglu_rows(const void *x, const int32_t *row_token, int64_t T, const void *b, void *h,
                                     const int64_t *batch_sizes, int64_t rows, int E, int64_t K, int64_t I, int dtype,
-                                    void *state, void *workspace, size_t workspace_bytes, void *stream) {
+                                    void *state, void *workspace, size_t workspace_bytes,
+                                    const int64_t *host_batch_sizes, void *stream) {
+    const HostSizes known(host_batch_sizes);
     DMOE_REQUIRE(dtype == DMOE_BF16, DMOE_ERR_DTYPE, "dmoe_gmm_swiglu_rows: dtype %d (bf16 only)", dtype);
     int rc = check_gmm("dmoe_gmm_swiglu_rows", x, b, h, batch_sizes, rows, E, K, I, 32);
     if (rc != DMOE_OK) return rc;
@@ -674,7 +700,8 @@ extern "C" int dmoe_gmm_swiglu_rows(const void *x, const int32_t *row_token, int
 
 extern "C" int dmoe_gmm_fp8(const void *a, const float *a_scale, const void *b, const float *b_scale, void *c,
                             const int64_t *batch_sizes, int64_t rows, int E, int64_t K, int64_t N, void *state,
-                            void *workspace, size_t workspace_bytes, void *stream) {
+                            void *workspace, size_t workspace_bytes, const int64_t *host_batch_sizes, void *stream) {
+    const HostSizes known(host_batch_sizes);
     int rc = check_gmm("dmoe_gmm_fp8", a, b, c, batch_sizes, rows, E, K, N, 16);
     if (rc != DMOE_OK) return rc;
     DMOE_REQUIRE(b_scale != nullptr && (rows == 0 || a_scale != nullptr), DMOE_ERR_ARG, "dmoe_gmm_fp8: null scales");
@@ -687,7 +714,9 @@ extern "C" int dmoe_gmm_fp8(const void *a, const float *a_scale, const void *b, 
 
 extern "C" int dmoe_gmm_fp8_swiglu(const void *a, const float *a_scale, const void *b, const float *b_scale, void *h,
                                    const int64_t *batch_sizes, int64_t rows, int E, int64_t K, int64_t I,
-                                   void *state, void *workspace, size_t workspace_bytes, void *stream) {
+                                   void *state, void *workspace, size_t workspace_bytes,
+                                   const int64_t *host_batch_sizes, void *stream) {
+    const HostSizes known(host_batch_sizes);
     int rc = check_gmm("dmoe_gmm_fp8_swiglu", a, b, h, batch_sizes, rows, E, K, I, 16);
     if (rc != DMOE_OK) return rc;
     DMOE_REQUIRE(b_scale != nullptr && (rows == 0 || a_scale != nullptr), DMOE_ERR_ARG, "dmoe_gmm_fp8_swiglu: null scales");

@@ -331,14 +331,28 @@ struct GmmLaunch {
     bool may_cut;      // the kernel cuts tiles along K when the launch has a workspace
     long long grid;    // workgroups
 };
+// The caller's copy of batch_sizes in host memory for the call that this thread is in, or nullptr: the reference keeps
+// the sizes on the host wherever it does not run its CUTLASS path (disagmoe/frontend/engine.py:377-380, 690-701).
+// With it the host knows the m-tiles of every tile height exactly; without it rows / tile_rows + E bounds them from above.
+extern thread_local const int64_t *t_host_sizes;
+inline long long m_tiles_of(const GmmArgs &args, int tile_rows) {
+    if (t_host_sizes == nullptr) return args.rows / tile_rows + args.E;
+    long long tiles = 0, left = args.rows;
+    for (int e = 0; e < args.E; ++e) {
+        long long n = t_host_sizes[e] < 0 ? 0 : t_host_sizes[e];
+        if (n > left) n = left;                         // as the kernels clamp them
+        left -= n;
+        tiles += (n + tile_rows - 1) / tile_rows;
+    }
+    return tiles;
+}
 // Workgroups of a persistent launch: one per compute unit, fewer when the tiles (or, where tiles may be cut along a K
 // long enough for two pieces, their pieces) do not fill them; whole rows of XCDs, the tile order is XCD-aware only then.
-// The host does not know how the rows split over the experts: rows / tile_rows + E bounds the m-tiles from above.
 inline long long launch_grid(const GmmArgs &args, int tile_rows, bool swiglu, int stage_k, bool may_cut, int cus) {
     const int n_out = swiglu ? args.N / 2 : args.N;
     const int bno = swiglu ? 128 : 256;
     const long long n_tiles = (n_out + bno - 1) / bno;
-    long long pieces = (args.rows / tile_rows + args.E) * n_tiles;
+    long long pieces = m_tiles_of(args, tile_rows) * n_tiles;
     if (may_cut && args.arrive != nullptr && args.K / stage_k >= 2 * kMinPieceStagesIdle) pieces *= kMaxSplit;
     long long grid = cus;
     if (pieces < grid) grid = pieces;

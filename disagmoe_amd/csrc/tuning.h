@@ -9,5 +9,6 @@ extern "C" int dmoe_gmm_tune(int variant);
 
 // What a launch with these shapes would run: kernel, tile rows, grid and (with the batch sizes in host memory) the
 // split of the last round, as the library itself derives them; for the benchmark's labels and the tests' expectations.
-extern "C" int dmoe_gmm_plan(const int64_t *host_batch_sizes, int64_t rows, int E, int64_t K, int64_t N, int trans_b,
-                             int swiglu, int dtype, size_t workspace_bytes, int64_t *out);
+// launch_has_sizes: the launch is given the host sizes as well (host_batch_sizes of dmoe_gmm*) and decides with them.
+extern "C" int dmoe_gmm_plan(const int64_t *host_batch_sizes, int launch_has_sizes, int64_t rows, int E, int64_t K, int64_t N,
+                             int trans_b, int swiglu, int dtype, size_t workspace_bytes, int64_t *out);

@@ -28,6 +28,8 @@ class ExpertsExecutor:
         ]
 
     def execute(self, layer_id: int, num_tokens: int, hidden_states: torch.Tensor,
-                batch_sizes: torch.Tensor) -> torch.Tensor:
+                batch_sizes: torch.Tensor, host_batch_sizes: Optional[torch.Tensor] = None) -> torch.Tensor:
         operator = self.operators[self.layer_mappings[layer_id]]
-        return operator.forward(num_tokens, hidden_states, batch_sizes)
+        if host_batch_sizes is None:
+            return operator.forward(num_tokens, hidden_states, batch_sizes)
+        return operator.forward(num_tokens, hidden_states, batch_sizes, host_batch_sizes=host_batch_sizes)

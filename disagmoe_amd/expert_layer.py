@@ -149,7 +149,8 @@ class ExpertWorker:
         if self._overflow is not None:
             mappings = self._overflow[0].to(dev, non_blocking=True)
             weights = self._overflow[1].to(dev, non_blocking=True) if self._overflow[1] is not None else None
-            output = self.executor.execute(layer_id, rows, input_tensor, self.static_batch_sizes)
+            output = self.executor.execute(layer_id, rows, input_tensor, self.static_batch_sizes,
+                                               host_batch_sizes=self._host_batch_sizes)
         else:
             mappings = self.static_mappings[:rows]
             weights = self.static_weights[:rows] if self.top_k > 1 else None
@@ -158,7 +159,8 @@ class ExpertWorker:
                 mappings.copy_(self._host_mappings[:rows], non_blocking=True)
                 if weights is not None:
                     weights.copy_(self._host_weights[:rows], non_blocking=True)
-                output = self.executor.execute(layer_id, rows, input_tensor, self.static_batch_sizes)
+                output = self.executor.execute(layer_id, rows, input_tensor, self.static_batch_sizes,
+                                               host_batch_sizes=self._host_batch_sizes)
             else:
                 # the mapping and the weights travel on the upload stream while the FFN runs (engine.py:717-729)
                 self.h2d_stream.wait_event(self._consumed)
@@ -167,7 +169,8 @@ class ExpertWorker:
                     if weights is not None:
                         weights.copy_(self._host_weights[:rows], non_blocking=True)
                     self._uploaded.record(self.h2d_stream)
-                output = self.executor.execute(layer_id, rows, input_tensor, self.static_batch_sizes)
+                output = self.executor.execute(layer_id, rows, input_tensor, self.static_batch_sizes,
+                                               host_batch_sizes=self._host_batch_sizes)
                 cur.wait_event(self._uploaded)
         output = memory.permute_tokens_cuda(output, mappings, row_scale=weights)
         if not torch.cuda.is_current_stream_capturing():

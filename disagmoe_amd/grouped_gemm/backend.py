@@ -77,9 +77,23 @@ def shared_workspace(device: torch.device, stream: Optional[int] = None) -> torc
     return _default_pair(device, _stream(device) if stream is None else stream)[1]
 
 
-def _state_args(device: torch.device, workspace: Optional[torch.Tensor], arguments_ptr: Optional[int], stream: int):
-    """The three state arguments of a dmoe_gmm* call and its stream."""
-    return (*_state_triple(device, workspace, arguments_ptr, stream), stream)
+def _state_args(device: torch.device, workspace: Optional[torch.Tensor], arguments_ptr: Optional[int], stream: int,
+                host_sizes: Optional[torch.Tensor] = None):
+    """The trailing arguments of a dmoe_gmm* call: state block, workspace and its size, the host copy of the sizes
+    (or NULL), the stream."""
+    return (*_state_triple(device, workspace, arguments_ptr, stream),
+            None if host_sizes is None else host_sizes.data_ptr(), stream)
+
+
+def _host_sizes(batch_sizes: torch.Tensor, host_batch_sizes: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
+    """The sizes in host memory, if the caller has them there: ``batch_sizes`` itself when it is a host tensor (what the
+    reference passes off its CUTLASS path, engine.py:377-380,690-701), or the copy given beside a device tensor.
+    The library then counts the tiles of a launch instead of estimating them (include/dmoe.h)."""
+    h = host_batch_sizes if host_batch_sizes is not None else (batch_sizes if batch_sizes.device.type == "cpu" else None)
+    if h is None or torch.cuda.is_current_stream_capturing():
+        return None     # (a recorded launch is replayed on other batches: it keeps the plan that fits any of them)
+    assert h.device.type == "cpu" and h.dim() == 1 and h.numel() == batch_sizes.numel()
+    return h.to(dtype=torch.int64).contiguous()
 
 
 def _state_triple(device, workspace, arguments_ptr, stream):
@@ -110,19 +124,22 @@ KERNEL_NAMES = {0: "dmoe::gmm_kernel", 1: "dmoe::gmm_direct_kernel", 2: "dmoe::g
 
 
 def launch_plan(rows: int, num_experts: int, K: int, N: int, swiglu: bool = False, fp8: bool = False,
-                workspace_bytes: int = 0, batch_sizes=None, trans_b: bool = False) -> dict:
+                workspace_bytes: int = 0, batch_sizes=None, trans_b: bool = False, sizes_passed: bool = False) -> dict:
     """What the library would launch for these shapes (its own answer, dmoe_gmm_plan):
     kernel, tile rows, wavefronts, workgroups; with ``batch_sizes`` (host values) also the
     tiles, how many of them are cut along K into how many pieces, and the work items.
-    ``N`` is the number of result columns (``I`` for the swiglu form)."""
+    ``N`` is the number of result columns (``I`` for the swiglu form).  ``sizes_passed``: the
+    launch is given the sizes in host memory too (``host_batch_sizes`` or a host ``batch_sizes``
+    tensor) and decides tile rows and workgroups from them instead of from ``rows / E``."""
     out = (_lib.ctypes.c_int64 * 9)()
     sizes = None
     if batch_sizes is not None:
         vals = [int(v) for v in (batch_sizes.tolist() if torch.is_tensor(batch_sizes) else batch_sizes)]
         assert len(vals) == num_experts
         sizes = (_lib.ctypes.c_int64 * num_experts)(*vals)
-    _lib.call("dmoe_gmm_plan", sizes, int(rows), int(num_experts), int(K), int(N), 1 if trans_b else 0, 1 if swiglu else 0,
-              _lib.FP8_E4M3 if fp8 else _lib.BF16, int(workspace_bytes), out)
+    _lib.call("dmoe_gmm_plan", sizes, 1 if (sizes_passed and sizes is not None) else 0, int(rows), int(num_experts),
+              int(K), int(N), 1 if trans_b else 0, 1 if swiglu else 0, _lib.FP8_E4M3 if fp8 else _lib.BF16,
+              int(workspace_bytes), out)
     keys = ("kernel_id", "tile_rows", "wavefronts", "workgroups", "stage_k", "tiles", "cut_tiles", "pieces_per_cut_tile", "items")
     plan = dict(zip(keys, (int(v) for v in out)))
     plan["kernel"] = KERNEL_NAMES[plan["kernel_id"]]
@@ -141,7 +158,7 @@ def _check_operands(a: torch.Tensor, b: torch.Tensor, dtype: torch.dtype) -> tor
 
 def gmm(a: torch.Tensor, b: torch.Tensor, batch_sizes: torch.Tensor, trans_b: bool = False,
         c: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None,
-        arguments_ptr: Optional[int] = None) -> torch.Tensor:
+        arguments_ptr: Optional[int] = None, host_batch_sizes: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``c[o_e:o_e+n_e] = a[o_e:o_e+n_e] @ b[e]`` (``b[e].T`` with ``trans_b``),
     bf16 operands, fp32 accumulation, bf16 result.  ``c`` (optional) is a
     preallocated ``[>= rows, N]`` buffer written in place and returned
@@ -162,13 +179,14 @@ def gmm(a: torch.Tensor, b: torch.Tensor, batch_sizes: torch.Tensor, trans_b: bo
     bs = _sizes_on_device(batch_sizes, device)
     with torch.cuda.device(device):
         _lib.call("dmoe_gmm", a.data_ptr(), b.data_ptr(), c.data_ptr(), bs.data_ptr(), rows, E, K, N,
-                  1 if trans_b else 0, _lib.BF16, *_state_args(device, workspace, arguments_ptr, _stream(device)))
+                  1 if trans_b else 0, _lib.BF16, *_state_args(device, workspace, arguments_ptr, _stream(device),
+                               _host_sizes(batch_sizes, host_batch_sizes)))
     return c
 
 
 def gmm_swiglu(a: torch.Tensor, b: torch.Tensor, batch_sizes: torch.Tensor, trans_b: bool = False,
                c: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None,
-               arguments_ptr: Optional[int] = None) -> torch.Tensor:
+               arguments_ptr: Optional[int] = None, host_batch_sizes: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Gate-up projection with the activation fused: ``silu(u[:, :I]) * u[:, I:]``
     for ``u = gmm(a, b)``, ``b [E, K, 2I]`` (``[E, 2I, K]`` with ``trans_b``);
     returns ``[rows, I]``.  The two steps of experts.py:92-93 in one kernel, taken
@@ -187,13 +205,14 @@ def gmm_swiglu(a: torch.Tensor, b: torch.Tensor, batch_sizes: torch.Tensor, tran
     bs = _sizes_on_device(batch_sizes, device)
     with torch.cuda.device(device):
         _lib.call("dmoe_gmm_swiglu", a.data_ptr(), b.data_ptr(), c.data_ptr(), bs.data_ptr(), rows, E, K, inter,
-                  1 if trans_b else 0, _lib.BF16, *_state_args(device, workspace, arguments_ptr, _stream(device)))
+                  1 if trans_b else 0, _lib.BF16, *_state_args(device, workspace, arguments_ptr, _stream(device),
+                               _host_sizes(batch_sizes, host_batch_sizes)))
     return c
 
 
 def gmm_swiglu_rows(x: torch.Tensor, row_token: torch.Tensor, b: torch.Tensor, batch_sizes: torch.Tensor,
                     c: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None,
-                    arguments_ptr: Optional[int] = None) -> torch.Tensor:
+                    arguments_ptr: Optional[int] = None, host_batch_sizes: Optional[torch.Tensor] = None) -> torch.Tensor:
     """:func:`gmm_swiglu` on rows fetched where they lie: row ``r`` of the product is row
     ``row_token[r]`` of ``x [T, K]`` (``ops.memory.route_tokens_with_sources``), so the permute
     in front of the FFN (engine.py:671-680) needs no launch.  ``b [E, K, 2I]``; returns
@@ -211,7 +230,8 @@ def gmm_swiglu_rows(x: torch.Tensor, row_token: torch.Tensor, b: torch.Tensor, b
     bs = _sizes_on_device(batch_sizes, device)
     with torch.cuda.device(device):
         _lib.call("dmoe_gmm_swiglu_rows", x.data_ptr(), row_token.data_ptr(), T, b.data_ptr(), c.data_ptr(), bs.data_ptr(),
-                  rows, E, K, inter, _lib.BF16, *_state_args(device, workspace, arguments_ptr, _stream(device)))
+                  rows, E, K, inter, _lib.BF16, *_state_args(device, workspace, arguments_ptr, _stream(device),
+                               _host_sizes(batch_sizes, host_batch_sizes)))
     return c
 
 
@@ -303,7 +323,7 @@ def _fp8_common(a, a_scale, b, b_scale):
 
 def gmm_fp8(a: torch.Tensor, a_scale: torch.Tensor, b: torch.Tensor, b_scale: torch.Tensor,
             batch_sizes: torch.Tensor, c: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None,
-            arguments_ptr: Optional[int] = None) -> torch.Tensor:
+            arguments_ptr: Optional[int] = None, host_batch_sizes: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``c = (a @ b[e].T) * a_scale[:, None] * b_scale[e][None, :]`` in bf16; ``a``
     fp8 ``[rows, K]``, ``b`` fp8 ``[E, N, K]``."""
     rows, K, E, N = _fp8_common(a, a_scale, b, b_scale)
@@ -312,13 +332,15 @@ def gmm_fp8(a: torch.Tensor, a_scale: torch.Tensor, b: torch.Tensor, b_scale: to
     bs = _sizes_on_device(batch_sizes, a.device)
     with torch.cuda.device(a.device):
         _lib.call("dmoe_gmm_fp8", a.data_ptr(), a_scale.data_ptr(), b.data_ptr(), b_scale.data_ptr(), c.data_ptr(),
-                  bs.data_ptr(), rows, E, K, N, *_state_args(a.device, workspace, arguments_ptr, _stream(a.device)))
+                  bs.data_ptr(), rows, E, K, N,
+                  *_state_args(a.device, workspace, arguments_ptr, _stream(a.device),
+                               _host_sizes(batch_sizes, host_batch_sizes)))
     return c
 
 
 def gmm_fp8_swiglu(a: torch.Tensor, a_scale: torch.Tensor, b: torch.Tensor, b_scale: torch.Tensor,
                    batch_sizes: torch.Tensor, c: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None,
-                   arguments_ptr: Optional[int] = None) -> torch.Tensor:
+                   arguments_ptr: Optional[int] = None, host_batch_sizes: Optional[torch.Tensor] = None) -> torch.Tensor:
     """fp8 gate-up projection with fused ``silu(gate) * up``; ``b`` fp8 ``[E, 2I,
     K]``; returns bf16 ``[rows, I]``."""
     rows, K, E, N2 = _fp8_common(a, a_scale, b, b_scale)
@@ -328,7 +350,9 @@ def gmm_fp8_swiglu(a: torch.Tensor, a_scale: torch.Tensor, b: torch.Tensor, b_sc
     bs = _sizes_on_device(batch_sizes, a.device)
     with torch.cuda.device(a.device):
         _lib.call("dmoe_gmm_fp8_swiglu", a.data_ptr(), a_scale.data_ptr(), b.data_ptr(), b_scale.data_ptr(),
-                  c.data_ptr(), bs.data_ptr(), rows, E, K, N2 // 2, *_state_args(a.device, workspace, arguments_ptr, _stream(a.device)))
+                  c.data_ptr(), bs.data_ptr(), rows, E, K, N2 // 2,
+                  *_state_args(a.device, workspace, arguments_ptr, _stream(a.device),
+                               _host_sizes(batch_sizes, host_batch_sizes)))
     return c
 
 

@@ -97,24 +97,28 @@ class MoEExperts(_GemmState, torch.nn.Module):
         # state block of this layer's launches and where their workspace comes from (experts.py:69-77)
         self._init_gemm_state(dev, getattr(self, "_workspace_arg", None), getattr(self, "_own_workspace_arg", False))
 
-    def forward(self, bs: int, hiddens: torch.Tensor, batch_sizes: torch.Tensor) -> torch.Tensor:
+    def forward(self, bs: int, hiddens: torch.Tensor, batch_sizes: torch.Tensor,
+                host_batch_sizes: Optional[torch.Tensor] = None) -> torch.Tensor:
         """``gmm(silu(u[:, :I]) * u[:, I:], w2)`` with ``u = gmm(hiddens, w13)``
         (experts.py:92-96); gate-up, SiLU and the product are one kernel.  Below
         ``max_batch_size`` rows the static buffers are used (the reference's
-        cached branch, :83-90)."""
-        ws = self._gemm_state()
+        cached branch, :83-90).  ``batch_sizes`` on the host (what the reference passes
+        off its CUTLASS path) or ``host_batch_sizes`` beside a device tensor let the
+        library count the launch's tiles instead of estimating them."""
+        ws = dict(self._gemm_state(), host_batch_sizes=host_batch_sizes)
         if self.enable_cache and bs <= self.gmm_cache_max_batch_size and hiddens.shape[0] <= self.cache_up.shape[0]:
             h = gg.gmm_swiglu(hiddens, self.w13_weight, batch_sizes, c=self.cache_up, **ws)[:hiddens.shape[0]]
             return gg.gmm(h, self.w2_weight, batch_sizes, c=self.cache_down, **ws)[:hiddens.shape[0]]
         h = gg.gmm_swiglu(hiddens, self.w13_weight, batch_sizes, **ws)
         return gg.gmm(h, self.w2_weight, batch_sizes, **ws)
 
-    def forward_rows(self, x: torch.Tensor, row_token: torch.Tensor, batch_sizes: torch.Tensor) -> torch.Tensor:
+    def forward_rows(self, x: torch.Tensor, row_token: torch.Tensor, batch_sizes: torch.Tensor,
+                     host_batch_sizes: Optional[torch.Tensor] = None) -> torch.Tensor:
         """:meth:`forward` on rows that are fetched where they lie: ``x [T, d]`` in token order
         and ``row_token [R]`` (``ops.memory.route_tokens_with_sources``) instead of the
         expert-sorted copy ``hiddens [R, d]``: the gate-up kernel reads row ``row_token[r]`` of
         ``x``, and the permute in front of the FFN (engine.py:671-680) is never launched."""
-        ws = self._gemm_state()
+        ws = dict(self._gemm_state(), host_batch_sizes=host_batch_sizes)
         h = gg.gmm_swiglu_rows(x, row_token, self.w13_weight, batch_sizes, **ws)
         return gg.gmm(h, self.w2_weight, batch_sizes, **ws)
 
@@ -143,12 +147,14 @@ class MoEExpertsSerial(MoEExperts):
         super().__init__(hidden_size, intermediate_size, num_experts, tp_size, enable_cutlass_cache=False,
                          max_batch_size=max_batch_size, **kwargs)
 
-    def forward(self, num_tokens: int, hiddens: torch.Tensor, batch_sizes: torch.Tensor) -> torch.Tensor:
+    def forward(self, num_tokens: int, hiddens: torch.Tensor, batch_sizes: torch.Tensor,
+                host_batch_sizes: Optional[torch.Tensor] = None) -> torch.Tensor:
         inter = self.intermediate_size
         results = []
         s = 0
         single = batch_sizes.shape[0] == 1
-        for i, n in enumerate(batch_sizes.tolist()):
+        # (the sizes on the host, if the caller has them there: no synchronisation then)
+        for i, n in enumerate((batch_sizes if host_batch_sizes is None else host_batch_sizes).tolist()):
             cur = hiddens if single else hiddens[s:s + n]
             gate = torch.matmul(cur, self.w13_weight[i, :, :inter])
             up = torch.matmul(cur, self.w13_weight[i, :, inter:])
@@ -175,13 +181,15 @@ class MoEExpertsFP8(_GemmState, torch.nn.Module):
         self.w2_scale = torch.nn.Parameter(s2, requires_grad=False)
         self._init_gemm_state(w13.device, workspace, own_workspace)
 
-    def forward(self, bs: int, hiddens: torch.Tensor, batch_sizes: torch.Tensor) -> torch.Tensor:
+    def forward(self, bs: int, hiddens: torch.Tensor, batch_sizes: torch.Tensor,
+                host_batch_sizes: Optional[torch.Tensor] = None) -> torch.Tensor:
         xq, xs = gg.quantize_rows(hiddens)
-        return self.forward_quantized(bs, xq, xs, batch_sizes)
+        return self.forward_quantized(bs, xq, xs, batch_sizes, host_batch_sizes)
 
-    def forward_quantized(self, bs: int, xq: torch.Tensor, xs: torch.Tensor, batch_sizes: torch.Tensor) -> torch.Tensor:
+    def forward_quantized(self, bs: int, xq: torch.Tensor, xs: torch.Tensor, batch_sizes: torch.Tensor,
+                          host_batch_sizes: Optional[torch.Tensor] = None) -> torch.Tensor:
         """The same on rows that arrive quantised (``ops.memory.permute_quantize``)."""
-        ws = self._gemm_state()
+        ws = dict(self._gemm_state(), host_batch_sizes=host_batch_sizes)
         h = gg.gmm_fp8_swiglu(xq, xs, self.w13_q, self.w13_scale, batch_sizes, **ws)
         hq, hs = gg.quantize_rows(h)
         return gg.gmm_fp8(hq, hs, self.w2_q, self.w2_scale, batch_sizes, **ws)

@@ -248,15 +248,26 @@ int dmoe_combine(const void *y, const void *mappings, int map_type, const float 
  * state == NULL: counters of the library's own, one set per stream (at most 64
  * streams per device), nothing is cut; refused with DMOE_ERR_WORKSPACE while
  * `stream` is being captured into a graph, whose replays may run beside anything.
+ *
+ * host_batch_sizes (may be NULL): the caller's copy of batch_sizes in HOST memory,
+ * read during the call only.  The reference keeps the sizes on the host wherever
+ * it does not run its CUTLASS path (disagmoe/frontend/engine.py:377-380, 690-701:
+ * get_expert_batch_sizes for the host, get_expert_batch_sizes_cuda for the device).
+ * With them the library counts the tiles of every tile height instead of
+ * estimating them from rows / E (tile height and grid of a skewed batch); the
+ * kernels still read the sizes on the device, so values that disagree with
+ * batch_sizes cost speed, never correctness.
  */
 #define DMOE_GMM_STATE_BYTES 33024
 int dmoe_gmm_workspace_bytes(int E, size_t *bytes);
 int dmoe_gmm(const void *a, const void *b, void *c, const int64_t *batch_sizes,
              int64_t rows, int E, int64_t K, int64_t N, int trans_b, int dtype,
-             void *state, void *workspace, size_t workspace_bytes, void *stream);
+             void *state, void *workspace, size_t workspace_bytes,
+             const int64_t *host_batch_sizes, void *stream);
 int dmoe_gmm_swiglu(const void *a, const void *b, void *h, const int64_t *batch_sizes,
                     int64_t rows, int E, int64_t K, int64_t I, int trans_b, int dtype,
-                    void *state, void *workspace, size_t workspace_bytes, void *stream);
+                    void *state, void *workspace, size_t workspace_bytes,
+                    const int64_t *host_batch_sizes, void *stream);
 
 /* dmoe_gmm_swiglu on rows that are fetched where they lie: row r of the product is row row_token[r] of x [T, K]
  * (dmoe_route_sources writes row_token).  The duplicating permute in front of the FFN
@@ -266,7 +277,8 @@ int dmoe_gmm_swiglu(const void *a, const void *b, void *h, const int64_t *batch_
  * for problems whose rows do not fill such tiles, dmoe_permute + dmoe_gmm_swiglu is the faster pair. */
 int dmoe_gmm_swiglu_rows(const void *x, const int32_t *row_token, int64_t T, const void *b, void *h,
                          const int64_t *batch_sizes, int64_t rows, int E, int64_t K, int64_t I, int dtype,
-                         void *state, void *workspace, size_t workspace_bytes, void *stream);
+                         void *state, void *workspace, size_t workspace_bytes,
+                         const int64_t *host_batch_sizes, void *stream);
 
 /* ---- fp8 (e4m3) path: no counterpart in the reference ---------------------
  * Per-row quantisation: q[r, :] = fp8(x[r, :] / s[r]), s[r] = absmax(x[r, :]) / 448
@@ -285,13 +297,15 @@ int dmoe_permute_quant(const void *in, void *q, float *scales, const void *mappi
  *   b  fp8 [E, N, K] with b_scale fp32 [E, N]     (per output channel)
  *   c  bf16 [rows, N] = (a @ b[e]^T) * a_scale[r] * b_scale[e, n]
  * K % 16 == 0.  The swiglu form takes b [E, 2I, K], b_scale [E, 2I] and writes
- * h bf16 [rows, I] as dmoe_gmm_swiglu does.  `state` and `workspace` as for dmoe_gmm. */
+ * h bf16 [rows, I] as dmoe_gmm_swiglu does.  `state`, `workspace` and `host_batch_sizes` as for dmoe_gmm. */
 int dmoe_gmm_fp8(const void *a, const float *a_scale, const void *b, const float *b_scale, void *c,
                  const int64_t *batch_sizes, int64_t rows, int E, int64_t K, int64_t N,
-                 void *state, void *workspace, size_t workspace_bytes, void *stream);
+                 void *state, void *workspace, size_t workspace_bytes,
+                 const int64_t *host_batch_sizes, void *stream);
 int dmoe_gmm_fp8_swiglu(const void *a, const float *a_scale, const void *b, const float *b_scale,
                         void *h, const int64_t *batch_sizes, int64_t rows, int E, int64_t K,
-                        int64_t I, void *state, void *workspace, size_t workspace_bytes, void *stream);
+                        int64_t I, void *state, void *workspace, size_t workspace_bytes,
+                        const int64_t *host_batch_sizes, void *stream);
 
 #ifdef __cplusplus
 }

@@ -49,9 +49,9 @@ def test_host_side_argument_errors():
     assert lib.dmoe_permute(None, None, None, 8, 4, 4, 8, 9, None, None) == -3
     assert lib.dmoe_permute(None, None, None, 8, 4, 4, 8, 0, None, None) == -1
     assert lib.dmoe_combine(None, None, 8, None, None, 4, 0, 8, 0, 0, None) == -1
-    assert lib.dmoe_gmm(None, None, None, None, 16, 8, 60, 64, 0, 0, None, None, 0, None) == -2      # K % 8
-    assert lib.dmoe_gmm(None, None, None, None, 16, 8, 64, 64, 0, 1, None, None, 0, None) == -3      # fp16 not supported
-    assert lib.dmoe_gmm_fp8(None, None, None, None, None, None, 16, 8, 72, 64, None, None, 0, None) == -2  # K % 16
+    assert lib.dmoe_gmm(None, None, None, None, 16, 8, 60, 64, 0, 0, None, None, 0, None, None) == -2      # K % 8
+    assert lib.dmoe_gmm(None, None, None, None, 16, 8, 64, 64, 0, 1, None, None, 0, None, None) == -3      # fp16 not supported
+    assert lib.dmoe_gmm_fp8(None, None, None, None, None, None, 16, 8, 72, 64, None, None, 0, None, None) == -2  # K % 16
     header = open(os.path.join(ROOT, "include", "dmoe.h")).read()
     assert f"#define DMOE_GMM_STATE_BYTES {_lib.GMM_STATE_BYTES}" in header
     assert "dmoe_gmm_tune" not in header and hasattr(lib, "dmoe_gmm_tune")      # a test hook, not public ABI

@@ -353,6 +353,45 @@ def test_gmm_swiglu_rows_equals_permute_then_gmm(T, k, E, K, I):
     assert int(gg._STATE_BLOCKS[ptr].count_nonzero()) == 0
 
 
+@pytest.mark.parametrize("swiglu", [False, True])
+@pytest.mark.parametrize("sizes", [[700] + [0] * 40 + [324] + [0] * 22,          # two experts hold everything
+                                   [40, 1, 0, 300, 0, 0, 7, 676],                  # skewed, 8 experts
+                                   [16] * 64])                                     # even: the estimate is right already
+def test_batch_sizes_on_the_host_shape_the_launch(sizes, swiglu):
+    """``batch_sizes`` as a host tensor (what the reference passes off its CUTLASS path, engine.py:377-380,690-701), or a
+    host copy beside the device tensor: the library counts the tiles instead of estimating them from rows / E.  Same
+    results as with device sizes only (to the tolerance: another tile height may cut another tail along K), the plan it
+    reports is the exact one, and host sizes that disagree with the device's cost nothing but speed."""
+    announce(test="gmm_host_sizes", sizes=sizes[:8], E=len(sizes), swiglu=swiglu)
+    E, K, N = len(sizes), 512, 768
+    R = sum(sizes)
+    bs = torch.tensor(sizes, dtype=torch.int64)
+    a = _rand((R, K), 31)
+    b = _rand((E, K, 2 * N if swiglu else N), 32, std=0.05)
+    ref = ffn.gmm(a, b, bs, out_dtype=torch.float32)
+    if swiglu:
+        ref = torch.nn.functional.silu(ref[:, :N]) * ref[:, N:]
+    run = gg.gmm_swiglu if swiglu else gg.gmm
+    a_d, b_d = a.to(dev()), b.to(dev())
+    out_dev = run(a_d, b_d, bs.to(dev()))
+    out_host = run(a_d, b_d, bs)                                          # a host tensor, as the reference passes it
+    out_both = run(a_d, b_d, bs.to(dev()), host_batch_sizes=bs)
+    wrong = torch.tensor(sizes[::-1], dtype=torch.int64)
+    out_wrong = run(a_d, b_d, bs.to(dev()), host_batch_sizes=wrong)       # the kernels read the device's sizes
+    for out in (out_dev, out_host, out_both, out_wrong):
+        assert max_rel_err(out, ref) <= TOL_BF16, max_rel_err(out, ref)
+    assert torch.equal(out_host, out_both)
+    est = gg.launch_plan(R, E, K, N, swiglu=swiglu, batch_sizes=bs)
+    exact = gg.launch_plan(R, E, K, N, swiglu=swiglu, batch_sizes=bs, sizes_passed=True)
+    n_tiles = -(-N // (128 if swiglu else 256))
+    for plan in (est, exact):
+        assert plan["tiles"] == sum(-(-n // plan["tile_rows"]) for n in sizes) * n_tiles, plan
+    # without the sizes the grid is sized for rows / tile_rows + E m-tiles, with them for the tiles there are
+    print(f"[plan] estimated {est['tile_rows']} rows x {est['workgroups']} workgroups, exact {exact['tile_rows']} x {exact['workgroups']}")
+    assert exact["workgroups"] <= est["workgroups"] or exact["tile_rows"] != est["tile_rows"], (est, exact)
+    assert exact["workgroups"] <= -(-exact["tiles"] // 8) * 8, exact
+
+
 def test_gmm_launches_on_two_streams_keep_their_own_state():
     # a recorded graph of a layer (its own state block and workspace) is replayed on one stream while 80 eager launches
     # with the module-wide pair of another stream run beside it; both give the bits of their serial runs
@@ -377,7 +416,7 @@ def test_gmm_launches_on_two_streams_keep_their_own_state():
         with torch.cuda.graph(torch.cuda.CUDAGraph(), stream=side):
             from disagmoe_amd import _lib
             _lib.call("dmoe_gmm", a.data_ptr(), b.data_ptr(), out.data_ptr(), sizes.data_ptr(), R, E, K, N, 0, _lib.BF16,
-                      None, None, 0, torch.cuda.current_stream().cuda_stream)
+                      None, None, 0, None, torch.cuda.current_stream().cuda_stream)
     torch.cuda.synchronize()
     eager = []
     for round_ in range(4):

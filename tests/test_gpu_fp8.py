@@ -273,6 +273,23 @@ def test_fp8_cut_launches_alternating_operands_on_one_state(swiglu, variant):
         gg.set_tile_variant(0)
 
 
+@pytest.mark.parametrize("swiglu", [False, True])
+def test_fp8_batch_sizes_on_the_host(swiglu):
+    """The fp8 launches with the sizes in host memory as well (a host ``batch_sizes`` tensor, or a copy beside the device
+    tensor): same results, whatever plan the exact tile counts lead to."""
+    announce(test="fp8_host_sizes", swiglu=swiglu)
+    sizes = [300, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 212, 0, 0, 0, 0]
+    ops, exact = _fp8_case(512, 384, sizes, swiglu, 41)
+    run = gg.gmm_fp8_swiglu if swiglu else gg.gmm_fp8
+    bs_host = torch.tensor(sizes, dtype=torch.int64)
+    out_dev = run(*ops)
+    out_host = run(*ops[:4], bs_host)
+    out_both = run(*ops, host_batch_sizes=bs_host)
+    for out in (out_dev, out_host, out_both):
+        assert max_rel_err(out, exact) <= 1e-2, max_rel_err(out, exact)
+    assert torch.equal(out_host, out_both)
+
+
 def test_two_fp8_graphs_replayed_on_two_streams():
     """Two fp8 layers, each recorded into a graph of its own on the same capture stream, replayed at the same time on
     two streams: each layer brings its own state block and workspace, so both give the bits of their serial runs."""

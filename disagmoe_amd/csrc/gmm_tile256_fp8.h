@@ -247,7 +247,11 @@ void gmm_tile256_fp8_kernel(const GmmArgs p) {
                 half_step(t, std::integral_constant<int, 1>{}, t + 1 < T);
             }
             if (wm == 0) __syncthreads();
-            if (!short_tile && wave == 0) full_step_ticks = ((long long)wall_clock64() - t_begin) / T;
+            if (!short_tile && wave == 0) {
+                // (the fastest full tile so far: a tile that was held up by something else must not set the pace)
+                const long long ticks = ((long long)wall_clock64() - t_begin) / T;
+                if (full_step_ticks == 0 || ticks < full_step_ticks) full_step_ticks = ticks;
+            }
 
             // a piece of a split tile: its sums go to the workspace, and the piece that arrives last adds all of them up
             if (cur_part >= 0 &&

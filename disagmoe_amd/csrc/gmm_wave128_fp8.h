@@ -11,8 +11,9 @@
 // operand fragments of a k-step stay in registers (each is read from LDS ONCE per k-step) and a k-step of the lane's
 // share of the global loads (16 x 16 bytes) is in flight in registers on top of the k-step that sits in LDS ahead.
 //
-//   * operands e4m3 bytes, K-contiguous on both sides, scales applied in the epilogue; the LDS image of a k-step and
-//     the operand reads are those of gmm_tile256_fp8.h (rows of 128 bytes, chunk c of row r at c ^ swizzle(r));
+//   * operands e4m3 bytes, K-contiguous on both sides, scales applied in the epilogue; rows of 128 bytes in LDS, read as
+//     in gmm_tile256_fp8.h (lane l: row l % 16, the 16-byte chunks l / 16 and l / 16 + 4), with a swizzle of its own
+//     that keeps a lane's two chunks 64 bytes apart (one address register per operand);
 //   * one wavefront per SIMD, so everything shares one instruction stream: a k-step is 64 MFMAs of 32 cycles, and the
 //     16 LDS writes, 16 global loads and 32 operand reads of a lane are placed one or two behind an MFMA each;
 //   * the 8 x 8 MFMAs of a k-step run as four quadrants of 4 x 4 fragments, (rows, columns) = (lo, lo) (lo, hi) (hi, hi)
@@ -24,6 +25,8 @@
 //     A piece m of k-step s + 2 to this one, and loads the piece 16 on into the registers just freed.  The barrier
 //     stands in front of MFMA 33: every read of this k-step's buffer has been issued by then (the last behind MFMA 27)
 //     and k-step s + 1 is complete in the other one;
+//   * more pieces in flight do not help: a ring of 24 (a k-step and a half, a period of six k-steps in the code) ran
+//     1.39 us per k-step against 1.33 with 16 on the same box;
 //   * the MFMAs are written as asm with the accumulators tied to the upper half of the register file; the operand
 //     loads are buffer loads (rows past an expert's end and columns past N read as zeros without touching memory) and
 //     all memory operations are ones the compiler counts (no hand-counted waits in this kernel).
@@ -74,31 +77,33 @@ void gmm_wave128_fp8_kernel(const GmmArgs p) {
     const int streams = (G % kXcds == 0) ? kXcds : 1;
     const bool drawer = tid == 0;
 
-    auto swizzle = [](int row) { return (((row >> 1) & 1) << 2) | (((row >> 2) & 1) << 1); };
+    // The LDS image of a k-step: rows of 128 bytes, the 16-byte chunk c of row r at c ^ swizzle(r).  The swizzle moves a
+    // chunk inside its half of the row only (rows 2 and 4 apart in different chunks, which is what keeps the 8 lanes of a
+    // cycle of ds_read_b128 on different banks), so a lane's two chunks g and g + 4 sit exactly 64 bytes apart and one
+    // address register serves both.
+    auto swizzle = [](int row) { return ((row >> 1) & 1) | (((row >> 2) & 1) << 1); };
     // ---- a lane's share of a k-step: piece i of A is the 16-byte chunk tid % 8 of tile row tid / 8 + 32 i, piece i of B
     // the same of column slot tid / 8 + 32 i; a wavefront's load instruction fetches 8 whole lines of 128 bytes ----
     const int pc_row = tid >> 3, pc_chunk = tid & 7;
     // where they go in a buffer: rows 32 apart share the swizzle, so piece i sits 4 KiB behind piece i - 1
     const int w_addr = pc_row * kStepK + ((pc_chunk ^ swizzle(pc_row)) << 4);
-    // ---- operand reads: lane l, row l % 16, chunks g and g + 4 (g = l / 16): the second sits 64 bytes from the first ----
+    // ---- operand reads: lane l, row l % 16, chunks g and g + 4 (g = l / 16) ----
     const int l16 = lane & 15, g16 = lane >> 4;
     const int rd = (g16 ^ swizzle(l16)) << 4;
-    // LDS addresses kept in registers: per buffer, where a lane's first and second 16 bytes of the first A fragment and of
-    // the first B fragment are, and where its first piece goes; everything else is a constant distance from one of them
-    // (the two buffers are more than an instruction's 64 KiB of offset apart)
-    const int fa0 = (wm * TM + l16) * kStepK + rd;
-    const int fb0 = kBufA + ((SWIGLU ? wn * (TN / 2) : wn * TN) + l16) * kStepK + rd;
-    const char *fa_lo[2] = {smem + fa0, smem + kBuf + fa0};
-    const char *fa_hi[2] = {smem + (fa0 ^ 64), smem + kBuf + (fa0 ^ 64)};
-    const char *fb_lo[2] = {smem + fb0, smem + kBuf + fb0};
-    const char *fb_hi[2] = {smem + (fb0 ^ 64), smem + kBuf + (fb0 ^ 64)};
-    char *w_at[2] = {smem + w_addr, smem + kBuf + w_addr};
+    // LDS: [A of buffer 0][A of buffer 1][B of buffer 0][B of buffer 1], 32 KiB each, so that one address register per
+    // operand reaches both buffers with an instruction's 64 KiB of offset: four registers in all (reads of A and of B,
+    // writes of A and of B pieces).
+    constexpr int kBufStride = kBufA;                    // from an operand's buffer 0 to its buffer 1
+    constexpr int kRegionB = 2 * kBufA;                  // where the B buffers start
+    const char *fa_at = smem + (wm * TM + l16) * kStepK + rd;
+    const char *fb_at = smem + kRegionB + ((SWIGLU ? wn * (TN / 2) : wn * TN) + l16) * kStepK + rd;
+    char *wa_at = smem + w_addr, *wb_at = smem + kRegionB + w_addr;
     auto fb_dist = [](int j) {   // bytes from fragment 0 to fragment j
         return (SWIGLU ? ((j < FN / 2) ? j * 16 : kDN / 2 + (j - FN / 2) * 16) : j * 16) * kStepK;
     };
-    auto read32 = [](const char *lo, const char *hi, int dist) {   // a lane's 32 bytes of a fragment
-        const u32x4 x0 = *(const u32x4 *)(lo + dist);
-        const u32x4 x1 = *(const u32x4 *)(hi + dist);
+    auto read32 = [](const char *at, int dist) {          // a lane's 32 bytes of a fragment
+        const u32x4 x0 = *(const u32x4 *)(at + dist);
+        const u32x4 x1 = *(const u32x4 *)(at + dist + 64);
         return i32x8{(int)x0[0], (int)x0[1], (int)x0[2], (int)x0[3], (int)x1[0], (int)x1[1], (int)x1[2], (int)x1[3]};
     };
 
@@ -148,7 +153,7 @@ void gmm_wave128_fp8_kernel(const GmmArgs p) {
         return __builtin_amdgcn_raw_buffer_load_b128(k < kPieces ? a_buf : b_buf, lane_off + dist, 0, 0);
     };
     auto store_piece = [&](int buf, int k, const u32x4 &v) {
-        *(u32x4 *)(w_at[buf] + (k < kPieces ? 0 : kBufA) + (k % kPieces) * (32 * kStepK)) = v;
+        *(u32x4 *)((k < kPieces ? wa_at : wb_at) + buf * kBufStride + (k % kPieces) * (32 * kStepK)) = v;
     };
 
     unsigned int draw = 0;
@@ -182,8 +187,8 @@ void gmm_wave128_fp8_kernel(const GmmArgs p) {
         i32x8 fa[FM], fb[FN];
 #pragma unroll
         for (int x = 0; x < 4; ++x) {
-            fa[x] = read32(fa_lo[0], fa_hi[0], x * (16 * kStepK));
-            fb[x] = read32(fb_lo[0], fb_hi[0], fb_dist(x));
+            fa[x] = read32(fa_at, x * (16 * kStepK));
+            fb[x] = read32(fb_at, fb_dist(x));
         }
 
         // K-step s of the item; kPhase fixes the LDS buffer (s % 2), the order of the quadrants and where the ring of
@@ -208,22 +213,22 @@ void gmm_wave128_fp8_kernel(const GmmArgs p) {
                 // B, the half this k-step's second quadrant starts with (its registers were in use to the last k-step's end)
                 if constexpr (t < 16 && t % 4 == 0) {
                     constexpr int jj = (kPar == 0 ? 4 : 0) + t / 4;
-                    fb[jj] = read32(fb_lo[kPar], fb_hi[kPar], fb_dist(jj));
+                    fb[jj] = read32(fb_at, kPar * kBufStride + fb_dist(jj));
                 }
                 // A, rows 4 .. 7 of this k-step
                 if constexpr (t >= 15 && t < 31 && t % 4 == 3) {
                     constexpr int ii = 4 + (t - 15) / 4;
-                    fa[ii] = read32(fa_lo[kPar], fa_hi[kPar], ii * (16 * kStepK));
+                    fa[ii] = read32(fa_at, kPar * kBufStride + ii * (16 * kStepK));
                 }
                 // A, rows 0 .. 3 of the next k-step (behind the barrier: it is all in LDS then)
                 if constexpr (t >= 34 && t < 50 && t % 4 == 2) {
                     constexpr int ii = (t - 34) / 4;
-                    fa[ii] = read32(fa_lo[kPar ^ 1], fa_hi[kPar ^ 1], ii * (16 * kStepK));
+                    fa[ii] = read32(fa_at, (kPar ^ 1) * kBufStride + ii * (16 * kStepK));
                 }
                 // B, the half the next k-step's first quadrant takes (done with here since slot 47)
                 if constexpr (t >= 48 && t % 4 == 0) {
                     constexpr int jj = (kPar == 0 ? 4 : 0) + (t - 48) / 4;
-                    fb[jj] = read32(fb_lo[kPar ^ 1], fb_hi[kPar ^ 1], fb_dist(jj));
+                    fb[jj] = read32(fb_at, (kPar ^ 1) * kBufStride + fb_dist(jj));
                 }
                 // pieces: B piece m of k-step s + 1 into the other buffer, A piece m of k-step s + 2 into this one (free
                 // behind the barrier); each one's registers then take the piece kFlight on
@@ -243,11 +248,28 @@ void gmm_wave128_fp8_kernel(const GmmArgs p) {
         // (pairs without a condition between them, the odd one out behind the loop: the compiler counts the loads between
         // a piece's load and its use along every path, and a k-step that may or may not run would make it wait too early)
         int s = 0;
-        for (; s + 1 < T; s += 2) {
-            kstep(s, std::integral_constant<int, 0>{});
-            kstep(s + 1, std::integral_constant<int, 1>{});
+        if constexpr (kFlight % 16 == 0) {
+            for (; s + 1 < T; s += 2) {
+                kstep(s, std::integral_constant<int, 0>{});
+                kstep(s + 1, std::integral_constant<int, 1>{});
+            }
+            if (s < T) kstep(s, std::integral_constant<int, 0>{});
+        } else {
+            // (the ring comes round every 3 k-steps, the buffers every 2: six k-steps are one period)
+            for (; s + 5 < T; s += 6) {
+                kstep(s, std::integral_constant<int, 0>{});
+                kstep(s + 1, std::integral_constant<int, 1>{});
+                kstep(s + 2, std::integral_constant<int, 2>{});
+                kstep(s + 3, std::integral_constant<int, 3>{});
+                kstep(s + 4, std::integral_constant<int, 4>{});
+                kstep(s + 5, std::integral_constant<int, 5>{});
+            }
+            if (s < T) kstep(s, std::integral_constant<int, 0>{});
+            if (s + 1 < T) kstep(s + 1, std::integral_constant<int, 1>{});
+            if (s + 2 < T) kstep(s + 2, std::integral_constant<int, 2>{});
+            if (s + 3 < T) kstep(s + 3, std::integral_constant<int, 3>{});
+            if (s + 4 < T) kstep(s + 4, std::integral_constant<int, 4>{});
         }
-        if (s < T) kstep(s, std::integral_constant<int, 0>{});
         // (the compiler does not know how long the MFMAs above take: the last of them has left the pipe long before the
         // first accumulator is read, 32 cycles after its issue; these wait states make sure of it)
         asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15");

@@ -311,9 +311,13 @@ void gmm_tile256_kernel(const GmmArgs p) {
                 static_for<0, FM>([&](auto i_tag) {
                     constexpr int i = decltype(i_tag)::value;
                     if (kGuard && i >= nfr) return;        // wave-uniform
+                    // (j back and forth: one operand of every MFMA is the one the MFMA before it had, which the chip's
+                    // power limit pays back as clock: 2.7 % on a loop of MFMAs alone, 0.7 % here)
 #pragma unroll
-                    for (int j = 0; j < FN; ++j)
+                    for (int jj = 0; jj < FN; ++jj) {
+                        const int j = (i & 1) ? FN - 1 - jj : jj;
                         acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fb[j], fa[i], acc[i][j], 0, 0, 0);
+                    }
                 });
                 __builtin_amdgcn_s_setprio(0);
                 if (kAlt && next && wm == 0) landed();

@@ -223,10 +223,13 @@ void gmm_tile256_fp8_kernel(const GmmArgs p) {
                 static_for<0, FM / 2>([&](auto i_tag) {
                     constexpr int i = h * (FM / 2) + decltype(i_tag)::value;
                     if (kGuard && i >= nfr) return;        // wave-uniform
+                    // (j back and forth, so that every MFMA shares an operand with the one before it: less energy)
 #pragma unroll
-                    for (int j = 0; j < FN; ++j)
+                    for (int jj = 0; jj < FN; ++jj) {
+                        const int j = (i & 1) ? FN - 1 - jj : jj;
                         acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb[j], fa[decltype(i_tag)::value], acc[i][j],
                                                                                      0, 0, 0, 0, 0, 0);
+                    }
                 });
                 __builtin_amdgcn_s_setprio(0);
                 if (wm == 0) {

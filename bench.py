@@ -27,10 +27,10 @@ PEAK_FP8_TFLOPS = 5000.0
 # Bytes per launch of the dominant kernel that crossed the L2 boundary, from rocprofv3 --pmc runs of this script
 # (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, the factors read off a 1 GiB copy in the same runs).  A bench run does not
 # measure them: they are read off the committed summaries named here.  None = not measured.
-MEASURED_TRAFFIC = {"C2": (3.634e9, "profiles/expert_layer_c2_hbm_traffic.md"),
+MEASURED_TRAFFIC = {"C2": (3.500e9, "profiles/expert_layer_c2_hbm_traffic.md"),
                     "C3": (1.911e9, "profiles/expert_layer_c5_c4_c3_hbm_traffic.md"),
-                    "C4": (1.423e9, "profiles/expert_layer_c5_c4_c3_hbm_traffic.md"),
-                    "C5": (11.099e9, "profiles/expert_layer_c5_c4_c3_hbm_traffic.md")}
+                    "C4": (1.418e9, "profiles/expert_layer_c5_c4_c3_hbm_traffic.md"),
+                    "C5": (12.069e9, "profiles/expert_layer_c5_c4_c3_hbm_traffic.md")}
 
 
 def _event_ms(fn, iters: int, warmup: int = 2, plug=None):
